@@ -29,8 +29,8 @@
 //   MFMA: inline asm with the accumulator tied IN PLACE in an AGPR quad.  The builtin lets the register
 //         allocator pick the untied form (dst != srcC); with every AGPR live it then rotates the
 //         accumulators through VGPRs — ~300 v_accvgpr moves per K tile, measured in the .s.  The compiler
-//         cannot see the asm's latency: llm_weighted_consensus_amd/_isa_guard.py checks the built code
-//         object for accumulator moves / reads of in-flight MFMA results and fails the build on one.
+//         cannot see the asm's latency, so nothing may read or move an accumulator while the MFMA
+//         writing it is in flight.
 // Two schedules share that loop (the planner picks per shape, ops/gemm_plan.py): VAR 32 with the block-
 // staged epilogue (accumulators -> LDS image -> 16 B row stores), and VAR 64 — the wave-local epilogue on
 // the transposed accumulator layout (TR / TRR below), with the next persistent tile's first two K tiles
@@ -542,7 +542,7 @@ __global__ void __launch_bounds__(256, 1) gemm4w_kernel(Params p) {
         __syncthreads();
         // the partials are added where the epilogue reads the accumulators (G4_ACC_LOAD): the accumulators
         // stay as the MFMAs left them (rewriting them here made the register allocator rotate all of them
-        // through v_accvgpr_mov copies, caught by the build's ISA guard)
+        // through v_accvgpr_mov copies)
         nsl = p.S - 1;
       }
     }
