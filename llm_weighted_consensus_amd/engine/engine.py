@@ -348,15 +348,20 @@ class LLMEngine:
         # behind an admission (0 = whole admission batches, then decode: the throughput bench's mode)
         self.chunked_prefill = int(chunked_prefill)
         self._mixed_tuned = False
-        if self.chunked_prefill and self.cfg.head_dim != 128:
+        # models whose own attention kernels read prompt portions from the paged cache take any head size
+        self.paged_prefill = bool(getattr(model, "paged_prefill", False))
+        if self.chunked_prefill and self.cfg.head_dim != 128 and not self.paged_prefill:
             raise ValueError("chunked prefill: the paged-KV prefill kernel is built for head_dim 128")
         self.prefilling: List[SequenceGroup] = []
         self.width = (max_model_len + block_size - 1) // block_size
         if num_blocks is None:
             free, _total = torch.cuda.mem_get_info(self.device)
-            per = KVCache.bytes_per_block(self.cfg, block_size)
+            per = (model.bytes_per_block(block_size) if hasattr(model, "bytes_per_block")
+                   else KVCache.bytes_per_block(self.cfg, block_size))
             num_blocks = max(64, int(free * kv_memory_fraction) // per)
-        self.cache = KVCache(self.cfg, num_blocks, block_size, self.device)
+        # a model with a cache layout of its own (layers of different key / value sizes) builds it itself
+        self.cache = (model.new_cache(num_blocks, block_size) if hasattr(model, "new_cache")
+                      else KVCache(self.cfg, num_blocks, block_size, self.device))
         self.bm = BlockManager(num_blocks, block_size)
         # cross-request prefix cache (C++ block manager): prompts that start with an already computed
         # token prefix (the shared messages of a score request's voters, a repeated conversation) reuse
@@ -371,7 +376,7 @@ class LLMEngine:
         # split-K factor of the plain paged-decode kernel (None: chosen per batch bucket)
         self.decode_splits = decode_splits
         self.use_graphs = use_graphs
-        self.prefix_sharing = prefix_sharing
+        self.prefix_sharing = prefix_sharing and getattr(model, "supports_cascade", True)
         # decode batches >= this bucket use the cascade (shared-prompt) attention kernel; smaller ones
         # the split-K kernel, which spreads a few long contexts over more workgroups
         self.cascade_min_batch = cascade_min_batch
@@ -478,6 +483,100 @@ class LLMEngine:
             self.step()
         return [[list(s.tokens) for s in g.seqs] for g in groups]
 
+    # ------------------------------------------------------------------ given-token steps (trace replay, scoring)
+    def step_tokens(self, entries, end=()) -> Optional[torch.Tensor]:
+        """One engine step over GIVEN tokens instead of sampled ones: ``entries`` = [(key, tokens, want)], the
+        next tokens of each named sequence (admitted at its first entry; it may sit a step out) and the indices
+        among them whose logits are wanted.  All entries are ONE batch through the model's mixed forward —
+        single next tokens of started sequences as decode rows, everything else as prompt portions — on the
+        engine's block manager and paged cache, exactly as :meth:`_mixed_step` feeds sampled decoding and
+        chunked prompts.  Sequences named in ``end`` are freed after the step (their blocks return to the
+        pool).  Returns fp32 logits [sum(len(want)), V] in entry order, or None when nothing is wanted.
+        Only between generation work (nothing running or in flight)."""
+        if self.running or self.inflight is not None or self.prefilling:
+            raise RuntimeError("step_tokens while generation is in progress")
+        if not hasattr(self.model, "forward_mixed"):
+            raise RuntimeError("the model has no mixed forward")
+        if not hasattr(self, "_given"):
+            self._given: Dict[object, int] = {}
+            self._given_ids = itertools.count(1)
+        dev, bm = self.device, self.bm
+        if not entries:
+            for key in end:
+                sid = self._given.pop(key, None)
+                if sid is not None:
+                    bm.free_sequence(sid)
+            return None
+        dec, por = [], []  # (entry index, seq id, tokens, want)
+        for ei, (key, toks, want) in enumerate(entries):
+            toks = [int(t) for t in toks]
+            if not toks:
+                raise ValueError(f"step_tokens: no tokens for {key!r}")
+            if any(t < 0 or t >= self.cfg.vocab_size for t in toks):
+                raise ValueError(f"step_tokens: token id out of range for {key!r}")
+            if any(w < 0 or w >= len(toks) for w in want):
+                raise ValueError(f"step_tokens: wanted index out of range for {key!r}")
+            sid = self._given.get(key)
+            if sid is None:
+                sid = self._given[key] = -(1 << 50) - next(self._given_ids)
+                bm.add_sequence(sid, 0)
+            if bm.length(sid) + len(toks) > self.max_model_len:
+                raise ValueError(f"step_tokens: {key!r} grows past max_model_len ({self.max_model_len})")
+            (dec if len(toks) == 1 and bm.length(sid) > 0 else por).append((ei, sid, toks, list(want)))
+        need = sum(-(-(bm.length(sid) + len(t)) // self.block_size) - len(bm.block_table(sid)) for _, sid, t, _ in dec + por)
+        if need > bm.num_free:
+            raise RuntimeError(f"step_tokens: the step needs {need} more KV blocks, {bm.num_free} are free")
+        B = len(dec)
+        toks_all: List[int] = []
+        pos: List[int] = []
+        slot_parts: List[np.ndarray] = []
+        row_of: Dict[Tuple[int, int], int] = {}
+        dec_in = None
+        if B:
+            bt = np.zeros((B, self.width), np.int32)
+            cl, sl, ps = np.zeros(B, np.int32), np.zeros(B, np.int32), np.zeros(B, np.int32)
+            prepare_decode_into(bm, [sid for _, sid, _, _ in dec], self.width, B, bt, cl, sl, ps)
+            for r, (ei, _sid, t, want) in enumerate(dec):
+                toks_all.append(t[0])
+                for w in want:
+                    row_of[(ei, w)] = r
+            pos.extend(ps.tolist())
+            slot_parts.append(sl)
+            dec_in = {"block_tables": _h2d(bt, torch.int32, dev), "ctx_lens": _h2d(cl, torch.int32, dev), "splits": 1}
+        chunk_in = None
+        if por:
+            cu, k_lens, tables = [0], [], []
+            for ei, sid, t, want in por:
+                a = int(bm.length(sid))
+                slot_parts.append(np.asarray([bm.append_token(sid) for _ in t], dtype=np.int32))
+                toks_all.extend(t)
+                pos.extend(range(a, a + len(t)))
+                for w in want:
+                    row_of[(ei, w)] = B + cu[-1] + w
+                cu.append(cu[-1] + len(t))
+                k_lens.append(a + len(t))
+                tables.append(list(bm.block_table(sid)))
+            chunk_in = self._portion_tables(tables, cu, k_lens)
+        copies = bm.take_copies()
+        if copies:
+            self.cache.copy_blocks(_h2d(copies, torch.int32, dev))
+        rows = [row_of[(ei, w)] for ei, (_k, _t, want) in enumerate(entries) for w in want]
+        out = None
+        # a step whose logits nobody wants still writes its rows' keys and values: it runs with one dummy row
+        logits = self.model.forward_mixed(_h2d(toks_all, torch.int32, dev), _h2d(pos, torch.int32, dev),
+                                          _h2d(np.concatenate(slot_parts), torch.int32, dev), self.cache, B, dec_in,
+                                          chunk_in, _h2d(rows or [0], torch.int64, dev),
+                                          **({"float_logits": True} if getattr(self.model, "float_logits", False) else {}))
+        if rows:
+            out = logits.float()
+        self.stats["prefill_tokens"] += len(toks_all) - B
+        self.stats["decode_tokens"] += B
+        for key in end:
+            sid = self._given.pop(key, None)
+            if sid is not None:
+                bm.free_sequence(sid)
+        return out
+
     # ------------------------------------------------------------------ scheduling
     def _group_reservation(self, g: SequenceGroup) -> int:
         bs = self.block_size
@@ -558,7 +657,7 @@ class LLMEngine:
             cu.append(cu[-1] + L - c)
             last.append(cu[-1] - 1)
         ctx = None
-        if any(cached):
+        if any(cached) and not self.paged_prefill:
             k_lens = [len(p) for p in prompts]
             ks = np.concatenate([slots_range(self.bm, pid, 0, L) for pid, L in zip(parents, k_lens)]).astype(np.int64)
             if ks.size and (ks.min() < 0 or ks.max() >= self.bm.num_blocks * self.block_size):
@@ -573,7 +672,13 @@ class LLMEngine:
         t_cu = _h2d(cu, torch.int32, dev)
         t_last = _h2d(last, torch.int64, dev)
         max_len = max(len(p) - c for p, c in zip(prompts, cached))
-        logits = self.model.prefill(t_tok, t_pos, t_slots, t_cu, max_len, t_last, self.cache, ctx=ctx)
+        if self.paged_prefill:
+            # whole prompts (or their uncached tails) as portions over the paged cache, the mixed step's route
+            k_lens = [len(p) for p in prompts]
+            chunk_in = self._portion_tables([self.bm.block_table(pid) for pid in parents], cu, k_lens)
+            logits = self.model.forward_mixed(t_tok, t_pos, t_slots, self.cache, 0, None, chunk_in, t_last)
+        else:
+            logits = self.model.prefill(t_tok, t_pos, t_slots, t_cu, max_len, t_last, self.cache, ctx=ctx)
         if use_cache:
             for pid, p in zip(parents, prompts):
                 self.bm.cache_prefix(pid, p)
@@ -602,7 +707,7 @@ class LLMEngine:
             blocks.extend(tab)
             nblocks.append(len(tab))
         idx = torch.tensor(blocks, dtype=torch.int64, device=self.device)
-        kv = self.cache.pool.index_select(2, idx)
+        kv = self.cache.take_blocks(idx)
         for pid in parents:
             self.bm.free_sequence(pid)
         return kv, logits, nblocks
@@ -622,9 +727,9 @@ class LLMEngine:
             parent = -g.id
             self.bm.add_sequence(parent, len(g.prompt_ids))
             tab = torch.tensor(list(self.bm.block_table(parent)), dtype=torch.int64, device=dev)
-            if kv.shape[2] != tab.numel():
-                raise ValueError(f"imported KV has {kv.shape[2]} blocks, prompt needs {tab.numel()}")
-            self.cache.pool.index_copy_(2, tab, kv)
+            if self.cache.num_exported(kv) != tab.numel():
+                raise ValueError(f"imported KV has {self.cache.num_exported(kv)} blocks, prompt needs {tab.numel()}")
+            self.cache.put_blocks(tab, kv)
             logits_of[g.id] = row
             g.prefilled = None  # drop the reference: the cache owns the data now
         return self._start_groups(groups, logits_of)
@@ -743,13 +848,7 @@ class LLMEngine:
             k_lens.append(e)
             tables.append(list(self.bm.block_table(-g.id)))
             last_rows.append(B + cu[-1] - 1)
-        wc = 2 * -(-max(k_lens) // 32)
-        bt_c = np.zeros((len(items), wc), np.int32)
-        for i, t in enumerate(tables):
-            bt_c[i, :len(t)] = t[:wc]
-        chunk_in = {"cu_q": _h2d(cu, torch.int32, dev), "block_tables": _h2d(bt_c, torch.int32, dev),
-                    "k_lens": _h2d(k_lens, torch.int32, dev), "max_q": max(e - a for _, a, e in items),
-                    "lens": ([e - a for _, a, e in items], k_lens)}
+        chunk_in = self._portion_tables(tables, cu, k_lens)
         copies = self.bm.take_copies()
         if copies:
             self.cache.copy_blocks(_h2d(copies, torch.int32, dev))
@@ -796,6 +895,22 @@ class LLMEngine:
             self.running.extend(children)
             self._comp_cache = (None, None)
         return events
+
+    def _portion_tables(self, tables, cu: List[int], k_lens: List[int]) -> dict:
+        """Device inputs of the paged prefill kernels for prompt portions: ``tables`` (one block table per
+        portion), ``cu`` (row offsets of the portions, [n + 1]) and ``k_lens`` (keys each portion sees: its
+        sequence's length after this step)."""
+        dev, bs = self.device, self.block_size
+        wc = 2 * -(-max(k_lens) // (2 * bs))
+        bt_c = np.zeros((len(tables), wc), np.int32)
+        for i, t in enumerate(tables):
+            t = list(t)
+            bt_c[i, :min(len(t), wc)] = t[:wc]
+        if bt_c.size and (bt_c.min() < 0 or bt_c.max() >= self.bm.num_blocks):
+            raise RuntimeError("prompt portion: block id out of range")
+        q_lens = [cu[i + 1] - cu[i] for i in range(len(tables))]
+        return {"cu_q": _h2d(cu, torch.int32, dev), "block_tables": _h2d(bt_c, torch.int32, dev),
+                "k_lens": _h2d(k_lens, torch.int32, dev), "max_q": max(q_lens), "lens": (q_lens, k_lens)}
 
     def _block_chain(self, g: SequenceGroup) -> List[int]:
         """Chained hashes of the prompt's full blocks (block i's hash covers tokens [0, 16(i+1))), computed once
@@ -1364,7 +1479,7 @@ class LLMEngine:
         blocks, tables, lens = self.bm.swap_out([s.id for s in live])
         dev = self.device
         if blocks:
-            kv = self.cache.pool.index_select(2, torch.tensor(blocks, dtype=torch.int64, device=dev))
+            kv = self.cache.take_blocks(torch.tensor(blocks, dtype=torch.int64, device=dev))
             host = torch.empty(kv.shape, dtype=kv.dtype, pin_memory=dev.type == "cuda")
             host.copy_(kv, non_blocking=True)  # stream-ordered before any later write to the freed blocks
         else:
@@ -1387,7 +1502,7 @@ class LLMEngine:
         block per sequence and the watermark)."""
         while self.swapped:
             rec = self.swapped[0]
-            n = rec.host.shape[2] if rec.host.dim() == 4 else 0
+            n = self.cache.num_exported(rec.host)
             need = self._group_reservation(rec.group)
             if (n + len(rec.seqs) + self.kv_watermark > self.bm.num_free
                     or (need > self.free_blocks_unreserved and (self.running or self.inflight is not None))):
@@ -1397,7 +1512,7 @@ class LLMEngine:
             if n:
                 dev = self.device
                 kv = rec.host.to(dev, non_blocking=True)
-                self.cache.pool.index_copy_(2, torch.tensor(phys, dtype=torch.int64, device=dev), kv)
+                self.cache.put_blocks(torch.tensor(phys, dtype=torch.int64, device=dev), kv)
             rec.group.reserved_blocks = need
             self.free_blocks_unreserved -= need
             self.running.extend(s for s in rec.seqs if not s.finished)

@@ -6,8 +6,10 @@ Small variants exist for tests.
 """
 from __future__ import annotations
 
+import json
 from dataclasses import dataclass, replace
-from typing import Optional
+from pathlib import Path
+from typing import Optional, Tuple
 
 
 @dataclass(frozen=True)
@@ -99,3 +101,124 @@ def encoder_config(name: str, **overrides) -> EncoderConfig:
         key = key + "-en-v1.5"
     cfg = ENCODERS[key]
     return replace(cfg, **overrides) if overrides else cfg
+
+
+# ---------------------------------------------------------------------------------------------
+# layer-list decoders: every layer names its own mixer and feed-forward (read from a model folder's config.json)
+
+
+@dataclass(frozen=True)
+class WindowAttentionSpec:
+    """A sliding-window attention mixer: H query heads over G key/value heads, key size ``dim`` and value size
+    ``vdim`` per head, a window of ``window`` positions (itself and window - 1 before it), the softmax ``scale``
+    and whether the layer takes part in the value blending across layers."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    window: int
+    scale: float
+    v_mix: bool = False
+
+    @property
+    def nq(self) -> int:
+        return self.heads * self.dim
+
+    @property
+    def nk(self) -> int:
+        return self.kv_heads * self.dim
+
+    @property
+    def nv(self) -> int:
+        return self.kv_heads * self.vdim
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    type: str                      # the mixer's kind ("attention")
+    mixer: WindowAttentionSpec
+    mlp_kind: Optional[str]        # "dense" or None (no feed-forward in this layer)
+    ff: int = 0
+
+
+@dataclass(frozen=True)
+class MadipelConfig:
+    """Madipel: parallel layers (one LayerNorm feeds the mixer and the feed-forward, x += m (mixer + ff)) over an
+    fp32 residual stream, sinusoidal positions added to the embedding, windowed attention with whole-projection
+    q/k RMS norms, per-head temperature and a logarithmic distance bias, xIELU feed-forwards, LayerNorm + scaled
+    logits at the output."""
+    name: str
+    vocab_size: int
+    hidden: int
+    layer_specs: Tuple[LayerSpec, ...]
+    norm_eps: float
+    residual_mult: float
+    logit_scale: float
+    bos_token_id: int = 1
+    eos_token_id: int = 2
+    sinpos_base: float = 10000.0   # fixed by the design
+
+    architecture = "Madipel"
+
+    # what the engine reads of a decoder config
+    @property
+    def layers(self) -> int:
+        return len(self.layer_specs)
+
+    @property
+    def heads(self) -> int:
+        return max(L.mixer.heads for L in self.layer_specs)
+
+    @property
+    def kv_heads(self) -> int:
+        return max(L.mixer.kv_heads for L in self.layer_specs)
+
+    @property
+    def head_dim(self) -> int:
+        return max(L.mixer.dim for L in self.layer_specs)
+
+    num_experts = 0
+
+    @classmethod
+    def from_dict(cls, c: dict, name: str = "madipel") -> "MadipelConfig":
+        specs = []
+        for L in c["layers"]:
+            if L["type"] != "attention":
+                raise ValueError(f"Madipel: unknown mixer type {L['type']!r}")
+            m = L["mixer"]
+            mixer = WindowAttentionSpec(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]),
+                                        vdim=int(m["vdim"]), window=int(m["mask"]["size"]), scale=float(m["scale"]),
+                                        v_mix=bool(m.get("v_mix", False)))
+            if mixer.heads % mixer.kv_heads:
+                raise ValueError("Madipel: heads must be a multiple of kv_heads")
+            mlp = L.get("mlp")
+            if mlp is not None and mlp.get("kind") != "dense":
+                raise ValueError(f"Madipel: unknown feed-forward kind {mlp.get('kind')!r}")
+            specs.append(LayerSpec(L["type"], mixer, None if mlp is None else "dense", 0 if mlp is None else int(mlp["ff"])))
+        return cls(name=name, vocab_size=int(c["vocab"]), hidden=int(c["width"]), layer_specs=tuple(specs),
+                   norm_eps=float(c["norm"]["eps"]), residual_mult=float(c["residual_mult"]),
+                   logit_scale=float(c["logit_scale"]))
+
+    def params(self) -> int:
+        d = self.hidden
+        n = 2 * self.vocab_size * d + 2 * d
+        for L in self.layer_specs:
+            m = L.mixer
+            n += 2 * d + d * (m.nq + m.nk + m.nv) + m.nq + m.nk + 1 + 3 * m.heads + d * m.heads * m.vdim
+            n += 2 * d * L.ff + (2 if L.mlp_kind else 0)
+        return n
+
+
+# config.json "architecture" -> config class of the layer-list decoders
+ARCHITECTURES = {"Madipel": MadipelConfig}
+
+
+def load_model_config(model_dir) -> object:
+    """The config object of a model folder (config.json with an "architecture" this framework knows)."""
+    path = Path(model_dir) / "config.json"
+    with open(path) as f:
+        c = json.load(f)
+    arch = c.get("architecture")
+    if arch not in ARCHITECTURES:
+        raise ValueError(f"{path}: unknown architecture {arch!r} (known: {sorted(ARCHITECTURES)})")
+    return ARCHITECTURES[arch].from_dict(c, name=Path(model_dir).name or arch.lower())

@@ -94,6 +94,18 @@ class KVCache:
         if pairs.numel():
             ops.kv_block_copy(self.pool.view(self.cfg.layers * 2, self.num_blocks, self.block_elems), pairs)
 
+    # whole blocks leaving and entering the pool (swap, prefill hand-over): one layout-private tensor
+    def take_blocks(self, idx: torch.Tensor) -> torch.Tensor:
+        """The contents of blocks ``idx`` (int64), every layer, K and V: [L, 2, n, block_elems]."""
+        return self.pool.index_select(2, idx)
+
+    def put_blocks(self, idx: torch.Tensor, data: torch.Tensor) -> None:
+        self.pool.index_copy_(2, idx, data)
+
+    @staticmethod
+    def num_exported(data: torch.Tensor) -> int:
+        return int(data.shape[2]) if data.dim() == 4 else 0
+
 
 class _NullCache:
     """Shape-only stand-in for KVCache when no KV is written (encode): one shared 1-block buffer."""

@@ -1,0 +1,247 @@
+"""Madipel decoder on the fp32-residual kernel set (``ops/res32.py``, ``csrc/kernels/res32``).
+
+A layer is PARALLEL: one LayerNorm (weight and bias) feeds both sublayers, ``x += m * (mixer(h) + ff(h))``, and the
+residual stream x stays fp32.  Per layer (T rows of a step: decode rows and prompt-portion rows alike):
+
+    h     = layernorm(x)                                   res32.layernorm (fp32 statistics)
+    proj  = h @ [Wq | Wk | Wv | Wup]^T                     ONE GEMM over the fused input-side weight
+    q, kv = whole-projection RMS norms, per-head scale,    res32.proj_norm_kv_write (fp32; k, v into the paged
+            value blending across layers, cache write       cache, q into an fp32 buffer)
+    attn  = windowed attention with the log distance bias  res32.window_attn -> columns [0, H*Dv) of `cat`
+    act   = xIELU(proj[:, up columns])                     res32.xielu       -> columns [H*Dv, H*Dv + ff) of `cat`
+    y     = cat @ [Wo | Wdown]^T                           ONE GEMM: mixer and feed-forward outputs summed in
+                                                           the accumulators
+    x    += m * y                                          res32.residual_add_scaled (fp32)
+
+Positions enter through the sinusoidal vector added to the embedding and through the attention's distance bias
+(no rotation).  The output is LayerNorm -> head GEMM -> logits * logit_scale (fp32).
+
+Value blending: the first layer whose config says ``v_mix`` publishes its values v0 (per token, this step's
+rows); every later such layer caches ``(1 - lam) v + lam v0``.  v0 lives only inside one forward.
+
+``dtype=torch.float32`` runs every GEMM, activation and the cache in true fp32 (exact mode); bf16 is the serving
+mode.  GEMMs are the vendor library's (torch -> hipBLASLt), as for the other decoders' untuned shapes.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from pathlib import Path
+from typing import Callable, List, Optional
+
+import torch
+import torch.nn.functional as F
+
+from ..ops import res32
+from .cache import PagedLayerCache
+from .config import MadipelConfig
+
+
+@dataclass
+class MadipelLayer:
+    norm_w: torch.Tensor
+    norm_b: torch.Tensor
+    w_in: torch.Tensor        # [nq + nk + nv + ff, d]: q | k | v | up rows
+    w_out: torch.Tensor       # [d, H*Dv + ff]: o | down columns
+    q_norm: torch.Tensor      # [nq]
+    k_norm: torch.Tensor      # [nk]
+    head_scale: torch.Tensor  # fp32 [H]: softmax scale * the head's temperature
+    r1: torch.Tensor          # fp32 [H]
+    r2: torch.Tensor          # fp32 [H]
+    vmix: torch.Tensor        # [1] blend weight (activation dtype)
+    act: Optional[torch.Tensor]  # [2] xIELU parameters, None without a feed-forward
+    vmode: int = 0            # 0 plain, 1 publishes v0, 2 blends with v0
+
+
+class MadipelModel:
+    paged_prefill = True      # whole prompts run as one portion over the paged cache (engine._run_prefill)
+    supports_cascade = False  # no shared-prefix cascade kernel for this attention
+    graph_safe = True
+    float_logits = True       # forward_mixed / decode return fp32 logits when asked (float_logits=True)
+
+    def __init__(self, cfg: MadipelConfig, device="cuda", dtype=torch.bfloat16, seed: int = 0,
+                 weights_path: Optional[str] = None, max_position: Optional[int] = None):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError("Madipel runs in bfloat16 or float32")
+        self.cfg, self.device, self.dtype = cfg, torch.device(device), dtype
+        if self.device.type != "cuda":
+            raise RuntimeError("Madipel runs on the GPU kernels only (no CPU path)")
+        if dtype == torch.float32:
+            torch.backends.cuda.matmul.allow_tf32 = False  # true fp32 products
+        mixing = [L.mixer.nv for L in cfg.layer_specs if L.mixer.v_mix]
+        if len(set(mixing)) > 1:
+            raise ValueError("Madipel: layers that blend values must share kv_heads * vdim")
+        self.inv_freq = res32.sinpos_inv_freq(cfg.hidden, cfg.sinpos_base, self.device)
+        raw = self._read(weights_path) if weights_path else self._random(seed)
+        self._assemble(raw)
+        # called with (layer index, residual stream) after every layer when set (bring-up, tests)
+        self.on_layer: Optional[Callable[[int, torch.Tensor], None]] = None
+
+    # ------------------------------------------------------------------ weights
+    def tensor_shapes(self) -> dict:
+        """name -> shape of every tensor of a checkpoint of this config."""
+        cfg, d = self.cfg, self.cfg.hidden
+        out = {"embed": (cfg.vocab_size, d), "final.norm": (d,), "final.norm.b": (d,), "head": (cfg.vocab_size, d)}
+        for i, L in enumerate(cfg.layer_specs):
+            m, p = L.mixer, f"l{i}."
+            out.update({p + "norm1": (d,), p + "norm1.b": (d,), p + "mix.q": (m.nq, d), p + "mix.k": (m.nk, d),
+                        p + "mix.v": (m.nv, d), p + "mix.q.norm": (m.nq,), p + "mix.k.norm": (m.nk,),
+                        p + "mix.vmix": (), p + "mix.r1": (m.heads,), p + "mix.r2": (m.heads,),
+                        p + "mix.temp": (m.heads,), p + "mix.o": (d, m.heads * m.vdim)})
+            if L.mlp_kind:
+                out.update({p + "mlp.up": (L.ff, d), p + "mlp.down": (d, L.ff), p + "mlp.act": (2,)})
+        return out
+
+    def _random(self, seed: int) -> dict:
+        """Random weights of the config's shapes (benchmarks, tests): bf16-representable values."""
+        g = torch.Generator(device="cpu")
+        g.manual_seed(seed)
+        d = self.cfg.hidden
+        out = {}
+        for name, shape in self.tensor_shapes().items():
+            leaf = name.split(".")[-1]
+            if name.endswith("norm1") or name.endswith("final.norm") or leaf == "norm":
+                t = 1.0 + 0.1 * torch.randn(shape, generator=g)
+            elif leaf == "b":
+                t = 0.05 * torch.randn(shape, generator=g)
+            elif leaf == "vmix":
+                t = torch.rand(shape, generator=g) * 0.5
+            elif leaf in ("r1", "r2"):
+                t = 0.2 + torch.rand(shape, generator=g)
+            elif leaf == "temp":
+                t = 0.75 + 0.5 * torch.rand(shape, generator=g)
+            elif leaf == "act":
+                t = torch.randn(shape, generator=g) * 0.5
+            elif name == "embed":
+                t = torch.randn(shape, generator=g)
+            else:
+                t = torch.randn(shape, generator=g) / math.sqrt(shape[-1] if len(shape) > 1 else d)
+            out[name] = t.to(torch.bfloat16)
+        return out
+
+    def _read(self, path: str) -> dict:
+        from safetensors.torch import load_file
+
+        p = Path(path)
+        files = sorted(p.glob("*.safetensors")) if p.is_dir() else [p]
+        if not files:
+            raise FileNotFoundError(f"no .safetensors under {path}")
+        sd = {}
+        for f in files:
+            sd.update(load_file(str(f), device="cpu"))
+        want = self.tensor_shapes()
+        for name, shape in want.items():
+            if name not in sd:
+                raise KeyError(f"{path}: tensor {name} missing")
+            if tuple(sd[name].shape) != tuple(shape):
+                raise ValueError(f"{path}: {name} has shape {tuple(sd[name].shape)}, the config says {tuple(shape)}")
+        return sd
+
+    def _assemble(self, sd: dict) -> None:
+        cfg, dev, dt = self.cfg, self.device, self.dtype
+
+        def t(name):
+            return sd[name].to(device=dev, dtype=dt).contiguous()
+
+        def f32(name):
+            return sd[name].to(device=dev, dtype=torch.float32).contiguous()
+
+        self.embed = t("embed")
+        self.final_w, self.final_b, self.head = t("final.norm"), t("final.norm.b"), t("head")
+        self.layers: List[MadipelLayer] = []
+        published = False
+        for i, L in enumerate(cfg.layer_specs):
+            m, p = L.mixer, f"l{i}."
+            rows = [t(p + "mix.q"), t(p + "mix.k"), t(p + "mix.v")]
+            cols = [t(p + "mix.o")]
+            if L.mlp_kind:
+                rows.append(t(p + "mlp.up"))
+                cols.append(t(p + "mlp.down"))
+            vmode = 0
+            if m.v_mix:
+                vmode, published = (2 if published else 1), True
+            self.layers.append(MadipelLayer(
+                norm_w=t(p + "norm1"), norm_b=t(p + "norm1.b"), w_in=torch.cat(rows, 0).contiguous(),
+                w_out=torch.cat(cols, 1).contiguous(), q_norm=t(p + "mix.q.norm"), k_norm=t(p + "mix.k.norm"),
+                head_scale=(f32(p + "mix.temp") * m.scale).contiguous(), r1=f32(p + "mix.r1"), r2=f32(p + "mix.r2"),
+                vmix=t(p + "mix.vmix").reshape(1), act=t(p + "mlp.act") if L.mlp_kind else None, vmode=vmode))
+
+    # ------------------------------------------------------------------ cache
+    def _layer_dims(self):
+        return [(L.mixer.nk, L.mixer.nv) for L in self.cfg.layer_specs]
+
+    def new_cache(self, num_blocks: int, block_size: int) -> PagedLayerCache:
+        return PagedLayerCache(self._layer_dims(), num_blocks, block_size, self.device, self.dtype)
+
+    def bytes_per_block(self, block_size: int) -> int:
+        return PagedLayerCache.elems_per_block(self._layer_dims(), block_size) * (4 if self.dtype == torch.float32 else 2)
+
+    # ------------------------------------------------------------------ forward
+    def _forward(self, tokens, positions, slots, cache: PagedLayerCache, attend) -> torch.Tensor:
+        """Every layer over the step's rows; ``attend(q, li, out)`` runs the attention of layer ``li`` into
+        ``out`` (a column slice).  Returns the fp32 residual stream [T, d]."""
+        cfg = self.cfg
+        T = tokens.shape[0]
+        x = res32.embed_sinpos(self.embed, tokens, positions, self.inv_freq)
+        v0 = None
+        for li, (S, L) in enumerate(zip(cfg.layer_specs, self.layers)):
+            m = S.mixer
+            h = res32.layernorm(x, L.norm_w, L.norm_b, cfg.norm_eps)
+            proj = F.linear(h, L.w_in)
+            if L.vmode and v0 is None:
+                v0 = torch.empty(T, m.nv, dtype=torch.float32, device=x.device)
+            q = res32.proj_norm_kv_write(proj, L.q_norm, L.k_norm, L.head_scale, slots, cache.k[li], cache.v[li],
+                                         m.heads, m.dim, cfg.norm_eps, lam=L.vmix, v0=v0, vmode=L.vmode)
+            no = m.heads * m.vdim
+            cat = torch.empty(T, no + S.ff, dtype=self.dtype, device=x.device)
+            attend(q, li, cat[:, :no])
+            if S.mlp_kind:
+                res32.xielu(proj[:, m.nq + m.nk + m.nv:], L.act, cat[:, no:])
+            res32.residual_add_scaled(x, F.linear(cat, L.w_out), cfg.residual_mult)
+            if self.on_layer is not None:
+                self.on_layer(li, x)
+        return x
+
+    def _logits(self, x: torch.Tensor, rows: Optional[torch.Tensor], float_logits: bool) -> torch.Tensor:
+        h = res32.layernorm(x, self.final_w, self.final_b, self.cfg.norm_eps, rows=rows)
+        lg = F.linear(h, self.head).float() * self.cfg.logit_scale
+        return lg if float_logits else lg.to(torch.bfloat16)
+
+    def _attend(self, cache, positions, tables, cu_q=None):
+        def run(q, li, out, rows=slice(None)):
+            m = self.cfg.layer_specs[li].mixer
+            L = self.layers[li]
+            res32.window_attn(q[rows], cache.k[li], cache.v[li], positions[rows], tables, L.r1, L.r2, m.window,
+                              out[rows], m.heads, m.kv_heads, cu_q=cu_q)
+        return run
+
+    def decode(self, tokens: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor, block_tables: torch.Tensor,
+               ctx_lens: torch.Tensor, cache: PagedLayerCache, num_splits: int = 1, cascade_tiles=None,
+               float_logits: bool = False) -> torch.Tensor:
+        """One decode step for B sequences -> logits [B, V]; device tensors only (hipGraph-capturable).  Row b
+        reads table row b; its key range ends at its own position."""
+        x = self._forward(tokens, positions, slots, cache, self._attend(cache, positions, block_tables))
+        return self._logits(x, None, float_logits)
+
+    def forward_mixed(self, tokens: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor, cache: PagedLayerCache,
+                      n_dec: int, dec: Optional[dict], chunk: Optional[dict], logit_rows: torch.Tensor,
+                      float_logits: bool = False) -> torch.Tensor:
+        """ONE forward over [n_dec decode rows || prompt-portion rows]: every projection is one GEMM over both;
+        the attention runs per part (decode rows: table row = row; portion rows: the item of ``chunk['cu_q']``),
+        both over the paged cache that this step's rows were just written to.  Logits of ``logit_rows``."""
+        T = tokens.shape[0]
+        dec_run = self._attend(cache, positions, dec["block_tables"]) if n_dec else None
+        chk_run = self._attend(cache, positions, chunk["block_tables"], cu_q=chunk["cu_q"]) if T > n_dec else None
+        # (the portion rows' cu_q counts from the first portion row: each part gets its own row slice)
+
+        def attend(q, li, out):
+            if dec_run is not None:
+                dec_run(q, li, out, slice(0, n_dec))
+            if chk_run is not None:
+                chk_run(q, li, out, slice(n_dec, T))
+
+        x = self._forward(tokens, positions, slots, cache, attend)
+        return self._logits(x, logit_rows, float_logits)
+
+    def prefill(self, tokens, positions, slots, cu_seqlens, max_seqlen, last_idx, cache, ctx=None):
+        raise RuntimeError("Madipel prefills through forward_mixed over the paged cache (paged_prefill)")
