@@ -393,7 +393,9 @@ class LLMEngine:
         self.waiting: Deque[SequenceGroup] = deque()
         self.running: List[Sequence] = []
         self.lock = threading.Lock()
-        V = self.cfg.vocab_size
+        # columns of the logits the model hands the sampler (a vocabulary that is no multiple of 32 is padded
+        # with -inf columns by its model: the sampler works on 32-column words)
+        self.logit_width = int(getattr(model, "logit_width", self.cfg.vocab_size))
         self.counts: Optional[torch.Tensor] = None  # [max_batch, V] int16, lazily
         self.free_count_rows = list(range(max_batch))
         self.bias: Optional[torch.Tensor] = None    # [max_batch, V] f32, lazily
@@ -1025,15 +1027,15 @@ class LLMEngine:
         p = s.params
         if p.uses_penalties:
             if self.counts is None:
-                self.counts = torch.zeros(self.max_batch, self.cfg.vocab_size, dtype=torch.int16, device=self.device)
+                self.counts = torch.zeros(self.max_batch, self.logit_width, dtype=torch.int16, device=self.device)
             s.count_row = self.free_count_rows.pop()
             self.counts[s.count_row].zero_()
         g = s.group
         if p.logit_bias and g.bias_row < 0:
             if self.bias is None:
-                self.bias = torch.zeros(self.max_batch, self.cfg.vocab_size, dtype=torch.float32, device=self.device)
+                self.bias = torch.zeros(self.max_batch, self.logit_width, dtype=torch.float32, device=self.device)
             g.bias_row = self.free_bias_rows.pop()
-            row = torch.zeros(self.cfg.vocab_size, dtype=torch.float32)
+            row = torch.zeros(self.logit_width, dtype=torch.float32)
             for k, v in p.logit_bias.items():
                 row[int(k)] = float(v)
             self.bias[g.bias_row].copy_(row)
@@ -1373,7 +1375,7 @@ class LLMEngine:
         uploads only the B row indices."""
         if self._mask_rows_of is None:
             self._mask_rows_of = {}
-            self._mask_table = torch.zeros(64, self.cfg.vocab_size // 32, dtype=torch.int32, device=self.device)
+            self._mask_table = torch.zeros(64, self.logit_width // 32, dtype=torch.int32, device=self.device)
         rows = np.full(len(seqs), -1, dtype=np.int32)
         new: List[Tuple[int, np.ndarray]] = []
         for i in cons:

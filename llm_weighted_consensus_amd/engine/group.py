@@ -725,24 +725,30 @@ def build_engine(spec: dict, wid: int):
     """Default worker factory: a decoder engine on ``spec['device']`` from a server model spec
     ({"arch", "weights": "random:<seed>" | path, "max_model_len", "max_batch", "kv_fraction", "fp8",
     "prefix_caching", "chunked_prefill", "constrained_logprobs", "tokenizer": path to a tokenizer.json}); MoE archs get the
-    Mixtral model."""
+    Mixtral model.  ``"model_dir"`` instead of ``"arch"``: a folder with config.json + safetensors whose
+    "architecture" picks the class (``models.registry``; ``"dtype"``: bfloat16 | float32 where the design has both)."""
     import torch
 
-    from ..models.config import decoder_config
     from ..models.llama import LlamaModel
+    from ..models.registry import DTYPES, load_model, resolve_config
     from .engine import LLMEngine
     from .tokenizer import load_tokenizer
 
     dev = torch.device("cuda", int(spec.get("device", 0)))
     torch.cuda.set_device(dev)
-    cfg = decoder_config(spec["arch"])
+    cfg = resolve_config(spec)
     w = spec.get("weights", "random:0")
     path, seed = (None, int(w.split(":", 1)[1])) if w.startswith("random:") else (w, 0)
     mlen = int(spec.get("max_model_len", 4096))
     tp = int(spec.get("tp", 1) or 1)
     kv_fraction = float(spec.get("kv_fraction", 0.85))
     num_blocks = None
-    if cfg.num_experts:
+    if spec.get("model_dir"):
+        if tp > 1:
+            raise ValueError("model_dir decoders run on one GPU")
+        model = load_model(spec["model_dir"], device=dev, dtype=DTYPES[spec.get("dtype", "bfloat16")], max_position=mlen + 64,
+                           random_seed=seed if w.startswith("random:") and "weights" in spec else None)
+    elif cfg.num_experts:
         from ..models.mixtral import MixtralModel
 
         tp_kw = {}
@@ -773,6 +779,7 @@ def build_engine(spec: dict, wid: int):
                      use_graphs=getattr(model, "graph_safe", True),
                      prefix_caching=bool(spec.get("prefix_caching", True)),
                      # the paged-KV prefill kernel of mixed steps is built for head_dim 128
-                     chunked_prefill=int(spec.get("chunked_prefill", 0)) if cfg.head_dim == 128 else 0,
+                     chunked_prefill=(int(spec.get("chunked_prefill", 0))
+                                      if cfg.head_dim == 128 or getattr(model, "paged_prefill", False) else 0),
                      constrained_logprobs=bool(spec.get("constrained_logprobs", False)),
                      kv_reserve_tokens=spec.get("kv_reserve_tokens", 256))

@@ -38,7 +38,7 @@ def main(argv=None) -> int:
     if not _build.RUNTIME_SO.exists():  # a fresh checkout: the host runtime (g++) first; kernels build on first use
         _build.build_runtime()
     from .engine import LLMEngine
-    from .tokenizer import ByteTokenizer
+    from .tokenizer import load_tokenizer
 
     if not torch.cuda.is_available():
         print("trace_run: no GPU visible", file=sys.stderr)
@@ -52,7 +52,7 @@ def main(argv=None) -> int:
     if not hasattr(model, "forward_mixed"):
         print("trace_run: this model has no mixed forward", file=sys.stderr)
         return 2
-    eng = LLMEngine(model, ByteTokenizer(model.cfg.vocab_size), block_size=bs, num_blocks=max_len // bs,
+    eng = LLMEngine(model, load_tokenizer({}, model.cfg.vocab_size), block_size=bs, num_blocks=max_len // bs,
                     max_batch=a.max_seqs, max_model_len=max_len, use_graphs=False, prefix_sharing=False, tune_gc=False)
     os.makedirs(a.out, exist_ok=True)
     for line in sys.stdin:

@@ -60,6 +60,28 @@ class ByteTokenizer:
         return list(text.encode("utf-8"))
 
 
+class IdTokenizer(ByteTokenizer):
+    """For vocabularies too small to hold the 256 bytes: every id is its own word (`` w<base-36 id>``), text is
+    encoded byte by byte modulo the vocabulary.  The last two ids are bos / eos."""
+
+    def __init__(self, vocab_size: int):
+        if vocab_size < 2:
+            raise ValueError("vocab too small")
+        self.vocab_size = vocab_size
+        self.bos_token_id, self.eos_token_id = vocab_size - 2, vocab_size - 1
+        self.special = {self.bos_token_id: "", self.eos_token_id: ""}
+
+    def encode(self, text: str, add_bos: bool = False) -> List[int]:
+        n = max(1, self.vocab_size - 2)
+        return ([self.bos_token_id] if add_bos else []) + [b % n for b in text.encode("utf-8")]
+
+    def token_bytes(self, tid: int) -> bytes:
+        return b"" if tid in self.special else (" w" + _b36(tid)).encode()
+
+    def ids_for_text(self, text: str) -> List[int]:
+        raise ValueError("the id tokenizer cannot spell text (constrained decoding needs a byte vocabulary)")
+
+
 class IncrementalDecoder:
     """Streams UTF-8 text out of token bytes, holding back incomplete multi-byte sequences."""
 
@@ -179,8 +201,10 @@ class HFTokenizer:
 def load_tokenizer(spec: dict, vocab_size: int, bos_token_id: Optional[int] = None,
                    eos_token_id: Optional[int] = None):
     """Server model spec -> tokenizer: ``"tokenizer": "/path/tokenizer.json"`` loads it, otherwise the
-    byte tokenizer over the model's vocabulary."""
+    byte tokenizer over the model's vocabulary (the id tokenizer below 258 ids)."""
     path = spec.get("tokenizer")
     if path:
         return HFTokenizer(path, bos_token_id, eos_token_id)
+    if vocab_size < 258:
+        return IdTokenizer(vocab_size)
     return ByteTokenizer(vocab_size, bos_token_id, eos_token_id)

@@ -71,6 +71,8 @@ class MadipelModel:
         mixing = [L.mixer.nv for L in cfg.layer_specs if L.mixer.v_mix]
         if len(set(mixing)) > 1:
             raise ValueError("Madipel: layers that blend values must share kv_heads * vdim")
+        # the sampler reads logits in words of 32 columns: other vocabularies get -inf columns up to the next 32
+        self.logit_width = -(-cfg.vocab_size // 32) * 32
         self.inv_freq = res32.sinpos_inv_freq(cfg.hidden, cfg.sinpos_base, self.device)
         raw = self._read(weights_path) if weights_path else self._random(seed)
         self._assemble(raw)
@@ -205,7 +207,14 @@ class MadipelModel:
     def _logits(self, x: torch.Tensor, rows: Optional[torch.Tensor], float_logits: bool) -> torch.Tensor:
         h = res32.layernorm(x, self.final_w, self.final_b, self.cfg.norm_eps, rows=rows)
         lg = F.linear(h, self.head).float() * self.cfg.logit_scale
-        return lg if float_logits else lg.to(torch.bfloat16)
+        if float_logits:
+            return lg
+        V, Vp = self.cfg.vocab_size, self.logit_width
+        if Vp == V:
+            return lg.to(torch.bfloat16)
+        out = torch.full((lg.shape[0], Vp), float("-inf"), dtype=torch.bfloat16, device=lg.device)
+        out[:, :V] = lg
+        return out
 
     def _attend(self, cache, positions, tables, cu_q=None):
         def run(q, li, out, rows=slice(None)):

@@ -9,6 +9,8 @@ variables configure the local engine:
                     "tp": T (MoE decoders, BASELINE config 5) serves each replica tensor-parallel over T
                     consecutive LWC_GPUS entries — one process per GPU, the IPC one-shot all-reduce (C3)
                     inside every forward, the ranks stepping in lockstep behind the replica's rank 0
+                    {"model_dir": <folder>, "dtype": "bfloat16" | "float32"} instead of "arch": a folder with
+                    config.json + safetensors; its "architecture" picks the decoder class (e.g. Madipel)
   LWC_EMBED_MODELS  JSON {name: {"arch": "bge-large-en-v1.5", "weights": "random:<seed>" | <path>}}
   LWC_GPU           device index for this process's engine (one process per GPU)
   LWC_GPUS          comma list of devices: serve each model through an EngineGroup (one worker process

@@ -30,7 +30,7 @@ def build_state(cfg: Config, chat_client=None) -> AppState:
         from ..embeddings.service import build_embedding_service
         from ..engine.service import EngineService
         from ..engine.tokenizer import load_tokenizer
-        from ..models.config import decoder_config
+        from ..models.registry import resolve_config
 
         if cfg.device == "cpu":
             if cfg.models:
@@ -42,7 +42,7 @@ def build_state(cfg: Config, chat_client=None) -> AppState:
         for name, spec in cfg.embed_models.items():
             embedders[name] = build_embedding_service(name, spec, dev)
         for name, spec in cfg.models.items():
-            dcfg = decoder_config(spec["arch"])
+            dcfg = resolve_config(spec)
             mlen = int(spec.get("max_model_len", 4096))
             if cfg.gpus:  # one worker process per listed GPU behind one front end (LWC_GPUS=0: a single worker)
                 from ..engine.group import EngineGroup
