@@ -16,6 +16,10 @@ int r32_residual_add_scaled(float*, const void*, float, long long, int, hipStrea
 int r32_window_attn(const float*, const void*, const void*, long long, long long, int, const int*, const int*, int,
                     const int*, int, const float*, const float*, int, void*, int, int, int, int, int, int, int,
                     hipStream_t);
+int r32_window_attn_mfma_ok(int, int);
+int r32_window_attn_mfma(const float*, const void*, const void*, long long, long long, int, const int*, const int*,
+                         const int*, int, int, const int*, int, const float*, int, void*, int, int, int, int, int,
+                         hipStream_t);
 }
 
 namespace {
@@ -170,6 +174,43 @@ void window_attn(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, c10
                        D, Dv, f, stream()), "window_attn");
 }
 
+bool window_attn_mfma_ok(int64_t D, int64_t Dv) { return r32_window_attn_mfma_ok((int)D, (int)Dv) != 0; }
+
+// Prompt portions on the matrix cores: bf16 caches, q fp32 [T, H*D], bias fp32 [H, window] (the distance bias by
+// i - j), cu_q / k_lens int32 per item (k_lens: the sequence's length after this step), max_q the longest portion.
+// Positions ascend by one along each item's rows.
+void window_attn_mfma(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, Tensor cu_q, Tensor k_lens,
+                      int64_t max_q, Tensor block_tables, Tensor bias, int64_t window, Tensor out, int64_t H, int64_t G) {
+  want(q, torch::kFloat32, "window_attn_mfma q");
+  want(positions, torch::kInt32, "window_attn_mfma positions");
+  want(block_tables, torch::kInt32, "window_attn_mfma block_tables");
+  want(cu_q, torch::kInt32, "window_attn_mfma cu_q");
+  want(k_lens, torch::kInt32, "window_attn_mfma k_lens");
+  want(bias, torch::kFloat32, "window_attn_mfma bias");
+  TORCH_CHECK(k_cache.dim() == 3 && v_cache.dim() == 3 && k_cache.is_cuda() && v_cache.is_cuda() && out.is_cuda() &&
+                  k_cache.scalar_type() == torch::kBFloat16 && v_cache.scalar_type() == torch::kBFloat16 &&
+                  out.scalar_type() == torch::kBFloat16, "window_attn_mfma: bf16 caches and out");
+  const int T = (int)positions.numel();
+  const int NB = (int)k_cache.size(0), BS = (int)k_cache.size(1), nk = (int)k_cache.size(2), nv = (int)v_cache.size(2);
+  TORCH_CHECK(G > 0 && H > 0 && H % G == 0 && nk % G == 0 && nv % G == 0, "window_attn_mfma: head counts");
+  const int D = nk / (int)G, Dv = nv / (int)G;
+  TORCH_CHECK(r32_window_attn_mfma_ok(D, Dv), "window_attn_mfma: sizes not built");
+  const int ldo = row_stride(out, "window_attn_mfma out");
+  TORCH_CHECK(v_cache.size(0) == NB && v_cache.size(1) == BS && k_cache.stride(2) == 1 && k_cache.stride(1) == nk &&
+                  v_cache.stride(2) == 1 && v_cache.stride(1) == nv && k_cache.stride(0) % 8 == 0 && v_cache.stride(0) % 8 == 0 &&
+                  ((uintptr_t)k_cache.data_ptr() & 15) == 0 && ((uintptr_t)v_cache.data_ptr() & 15) == 0,
+              "window_attn_mfma: cache layout");
+  const int items = (int)block_tables.size(0);
+  TORCH_CHECK(block_tables.dim() == 2 && cu_q.numel() == items + 1 && k_lens.numel() == items && max_q >= 1 &&
+                  q.numel() == (int64_t)T * H * D && out.size(0) == T && out.size(1) == H * Dv && window >= 1 &&
+                  bias.numel() == H * window, "window_attn_mfma: shapes disagree");
+  done(r32_window_attn_mfma(q.data_ptr<float>(), k_cache.data_ptr(), v_cache.data_ptr(), (long long)k_cache.stride(0),
+                            (long long)v_cache.stride(0), BS, positions.data_ptr<int>(), cu_q.data_ptr<int>(),
+                            k_lens.data_ptr<int>(), items, (int)max_q, block_tables.data_ptr<int>(),
+                            (int)block_tables.size(1), bias.data_ptr<float>(), (int)window, out.data_ptr(), ldo, (int)H, (int)G,
+                            D, Dv, stream()), "window_attn_mfma");
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -180,4 +221,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("xielu", &xielu);
   m.def("residual_add_scaled", &residual_add_scaled);
   m.def("window_attn", &window_attn);
+  m.def("window_attn_mfma", &window_attn_mfma);
+  m.def("window_attn_mfma_ok", &window_attn_mfma_ok);
 }

@@ -165,3 +165,226 @@ extern "C" int r32_window_attn(const float* q, const void* k_cache, const void* 
                                                      bt_width, r1, r2, window, (bf16_t*)out, ldo, H, G, D, Dv);
   return (int)hipGetLastError();
 }
+
+// ---------------------------------------------------------------------------------------------------------
+// window_attn_mfma_kernel: prompt portions on the matrix cores (bf16 cache, D = 32 ND, Dv = 16 NV).
+//
+// Workgroup = 4 waves = 64 consecutive query rows of one (item, head); wave w owns rows 16w .. 16w+15 and all
+// four walk the 32-key tiles of the rows' windows, staged through LDS (K row-major, V transposed so that a
+// lane's four consecutive keys of one value column are one 8-byte read).  mfma_f32_16x16x32_bf16, lane l:
+// r16 = l & 15, g = l >> 4:
+//   S^T = K Q^T : A = K rows from LDS, B = Q^T in registers; C reg r = S^T[key 4g + r][query r16], two 16-key
+//                 subtiles.  q is fp32: it enters as hi + lo bf16 halves (two MFMAs), so the scores keep fp32's
+//                 precision against the cache's bf16 keys.
+//   O  += P V   : A = the lane's own softmax weights (k slots 8g+e <-> keys {4g+e, 16+4g+e-4}), again as hi + lo
+//                 halves; B = V^T from LDS with the same key permutation; C reg r = O[query 4g + r][dv 16n + r16].
+// The distance bias comes from a table bias[h][i - j] (fp32, built once from r1, r2).  Online softmax in fp32;
+// masked scores never enter it (weights forced to 0), rows are finite-initialised.
+// Positions ascend by one along an item's rows (a portion of a prompt).
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+
+LWC_DEVICE float4v mfma16(const short8& a, const short8& b, const float4v& c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+struct WAttnMfmaParams {
+  const float* q;
+  const bf16_t* k_cache;
+  const bf16_t* v_cache;
+  long long kb_stride, vb_stride;
+  int block_size;
+  const int* positions;
+  const int* cu_q;
+  const int* k_lens;
+  int tiles_per_item;
+  const int* block_tables;
+  int bt_width;
+  const float* bias;  // [H, window]
+  int window;
+  bf16_t* out;
+  int ldo, H, G;
+};
+
+constexpr int kVPad = 40;  // keys per V^T row in LDS (32 + 8: rows stay 16-byte aligned, banks spread)
+
+template <int ND, int NV>
+__global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaParams p) {
+  constexpr int D = 32 * ND, DV = 16 * NV, KLD = D + 8;
+  __shared__ __attribute__((aligned(16))) bf16_t K_s[32 * KLD];
+  __shared__ __attribute__((aligned(16))) bf16_t Vt_s[DV * kVPad];
+  const int it = blockIdx.x / p.tiles_per_item, tile = blockIdx.x % p.tiles_per_item;
+  const int q_begin = p.cu_q[it], q_end = p.cu_q[it + 1];
+  const int row0 = q_begin + tile * 64;
+  if (row0 >= q_end) return;
+  const int h = blockIdx.y, H = p.H, g = h / (H / p.G), G = p.G;
+  const int nrows = min(64, q_end - row0);
+  const int k_len = p.k_lens[it];
+  const int pos0 = p.positions[row0], pos_last = p.positions[row0 + nrows - 1];
+  const int j_lo = max(0, pos0 - p.window + 1), j_hi = min(pos_last, k_len - 1);
+  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, r16 = lane & 15, g4 = lane >> 4;
+  const int* table = p.block_tables + (size_t)it * p.bt_width;
+  const int BS = p.block_size;
+
+  const int qrow = 16 * w + r16;
+  const bool q_valid = qrow < nrows;
+  const int i_q = q_valid ? p.positions[row0 + qrow] : -1;
+  short8 qhi[ND], qlo[ND];
+#pragma unroll
+  for (int kd = 0; kd < ND; ++kd) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float x = 0.f;
+      if (q_valid) x = p.q[((size_t)(row0 + qrow) * H + h) * D + kd * 32 + 8 * g4 + e];
+      const bf16_t hi = f2bf(x);
+      qhi[kd][e] = (short)hi;
+      qlo[kd][e] = (short)f2bf(x - bf2f(hi));
+    }
+  }
+  const int w_min = pos0 + 16 * w, w_max = min(pos0 + 16 * w + 15, pos_last);  // this wave's positions
+  const bool wave_live = 16 * w < nrows;
+
+  float4v O[NV];
+#pragma unroll
+  for (int n = 0; n < NV; ++n) O[n] = float4v{0.f, 0.f, 0.f, 0.f};
+  float m = -1e30f, l = 0.f;
+  const float* bias_h = p.bias + (size_t)h * p.window;
+
+  for (int kt = j_lo / 32; kt <= j_hi / 32; ++kt) {
+    __syncthreads();
+    for (int c = tid; c < 32 * (D / 8); c += 256) {
+      const int key = c / (D / 8), dc = c % (D / 8);
+      const int j = kt * 32 + key;
+      uint4v val = uint4v{0u, 0u, 0u, 0u};
+      if (j <= j_hi) {
+        const long long page = table[j / BS];
+        val = *reinterpret_cast<const uint4v*>(p.k_cache + page * p.kb_stride + ((long long)(j % BS) * G + g) * D + dc * 8);
+      }
+      *reinterpret_cast<uint4v*>(&K_s[key * KLD + dc * 8]) = val;
+    }
+    for (int c = tid; c < 32 * (DV / 8); c += 256) {
+      const int key = c & 31, dc = c >> 5;
+      const int j = kt * 32 + key;
+      uint4v val = uint4v{0u, 0u, 0u, 0u};
+      if (j <= j_hi) {
+        const long long page = table[j / BS];
+        val = *reinterpret_cast<const uint4v*>(p.v_cache + page * p.vb_stride + ((long long)(j % BS) * G + g) * DV + dc * 8);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        Vt_s[(dc * 8 + 2 * e) * kVPad + key] = (bf16_t)(val[e] & 0xffffu);
+        Vt_s[(dc * 8 + 2 * e + 1) * kVPad + key] = (bf16_t)(val[e] >> 16);
+      }
+    }
+    __syncthreads();
+    // the tile's keys [32 kt, 32 kt + 31] against this wave's rows: nothing visible -> nothing to do
+    if (!wave_live || kt * 32 > w_max || kt * 32 + 31 < w_min - p.window + 1) continue;
+
+    float4v sacc[2];
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      sacc[sub] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kd = 0; kd < ND; ++kd) {
+        const short8 a = *reinterpret_cast<const short8*>(&K_s[(sub * 16 + r16) * KLD + kd * 32 + 8 * g4]);
+        sacc[sub] = mfma16(a, qhi[kd], sacc[sub]);
+        sacc[sub] = mfma16(a, qlo[kd], sacc[sub]);
+      }
+    }
+    float s[8];
+    bool ok[8];
+    float mx = -1e30f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int j = kt * 32 + (e >> 2) * 16 + 4 * g4 + (e & 3);
+      const int dist = i_q - j;
+      ok[e] = q_valid && dist >= 0 && dist < p.window;
+      s[e] = ok[e] ? sacc[e >> 2][e & 3] - bias_h[dist] : -1e30f;
+      mx = fmaxf(mx, s[e]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float alpha = expf(m - m_new);
+    float pe[8], psum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      pe[e] = ok[e] ? expf(s[e] - m_new) : 0.f;
+      psum += pe[e];
+    }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * alpha + psum;
+    m = m_new;
+    short8 ph, pl;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const bf16_t hi = f2bf(pe[e]);
+      ph[e] = (short)hi;
+      pl[e] = (short)f2bf(pe[e] - bf2f(hi));
+    }
+    float ar[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) ar[r] = __shfl(alpha, 4 * g4 + r, 64);
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) O[n][r] *= ar[r];
+      const bf16_t* vrow = &Vt_s[(n * 16 + r16) * kVPad];
+      const short4v b0 = *reinterpret_cast<const short4v*>(vrow + 4 * g4);
+      const short4v b1 = *reinterpret_cast<const short4v*>(vrow + 16 + 4 * g4);
+      const short8 b = short8{b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+      O[n] = mfma16(ph, b, O[n]);
+      O[n] = mfma16(pl, b, O[n]);
+    }
+  }
+  if (!wave_live) return;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float lr = __shfl(l, 4 * g4 + r, 64);
+    const float inv = lr > 0.f ? 1.0f / lr : 0.f;
+    const int row = 16 * w + 4 * g4 + r;
+    if (row < nrows) {
+      bf16_t* orow = p.out + (size_t)(row0 + row) * p.ldo + (size_t)h * DV;
+#pragma unroll
+      for (int n = 0; n < NV; ++n) orow[n * 16 + r16] = f2bf(O[n][r] * inv);
+    }
+  }
+}
+
+template <int ND>
+int launch_mfma_nv(const WAttnMfmaParams& p, int nv, dim3 grid, hipStream_t s) {
+  switch (nv) {
+    case 2: window_attn_mfma_kernel<ND, 2><<<grid, 256, 0, s>>>(p); break;
+    case 4: window_attn_mfma_kernel<ND, 4><<<grid, 256, 0, s>>>(p); break;
+    case 8: window_attn_mfma_kernel<ND, 8><<<grid, 256, 0, s>>>(p); break;
+    default: return -1;
+  }
+  return (int)hipGetLastError();
+}
+
+// Whether the matrix-core kernel takes these sizes (bf16 cache only).
+extern "C" int r32_window_attn_mfma_ok(int D, int Dv) {
+  return (D == 32 || D == 64 || D == 128) && (Dv == 32 || Dv == 64 || Dv == 128);
+}
+
+extern "C" int r32_window_attn_mfma(const float* q, const void* k_cache, const void* v_cache, long long kb_stride,
+                                    long long vb_stride, int block_size, const int* positions, const int* cu_q,
+                                    const int* k_lens, int n_items, int max_q, const int* block_tables, int bt_width,
+                                    const float* bias, int window, void* out, int ldo, int H, int G, int D, int Dv,
+                                    hipStream_t s) {
+  if (n_items <= 0 || max_q <= 0) return 0;
+  if (!r32_window_attn_mfma_ok(D, Dv) || H % G != 0) return -1;
+  WAttnMfmaParams p;
+  p.q = q; p.k_cache = (const bf16_t*)k_cache; p.v_cache = (const bf16_t*)v_cache;
+  p.kb_stride = kb_stride; p.vb_stride = vb_stride; p.block_size = block_size; p.positions = positions;
+  p.cu_q = cu_q; p.k_lens = k_lens; p.tiles_per_item = (max_q + 63) / 64; p.block_tables = block_tables;
+  p.bt_width = bt_width; p.bias = bias; p.window = window; p.out = (bf16_t*)out; p.ldo = ldo; p.H = H; p.G = G;
+  const dim3 grid(n_items * p.tiles_per_item, H);
+  switch (D / 32) {
+    case 1: return launch_mfma_nv<1>(p, Dv / 16, grid, s);
+    case 2: return launch_mfma_nv<2>(p, Dv / 16, grid, s);
+    case 4: return launch_mfma_nv<4>(p, Dv / 16, grid, s);
+  }
+  return -1;
+}

@@ -51,6 +51,7 @@ class MadipelLayer:
     vmix: torch.Tensor        # [1] blend weight (activation dtype)
     act: Optional[torch.Tensor]  # [2] xIELU parameters, None without a feed-forward
     vmode: int = 0            # 0 plain, 1 publishes v0, 2 blends with v0
+    bias: Optional[torch.Tensor] = None  # fp32 [H, window] distance-bias table (matrix-core prompt kernel)
 
 
 class MadipelModel:
@@ -167,6 +168,9 @@ class MadipelModel:
                 w_out=torch.cat(cols, 1).contiguous(), q_norm=t(p + "mix.q.norm"), k_norm=t(p + "mix.k.norm"),
                 head_scale=(f32(p + "mix.temp") * m.scale).contiguous(), r1=f32(p + "mix.r1"), r2=f32(p + "mix.r2"),
                 vmix=t(p + "mix.vmix").reshape(1), act=t(p + "mlp.act") if L.mlp_kind else None, vmode=vmode))
+            Lw = self.layers[-1]
+            if dt == torch.bfloat16 and m.heads * m.window <= (1 << 26) and res32.kernels().window_attn_mfma_ok(m.dim, m.vdim):
+                Lw.bias = res32.distance_bias(Lw.r1, Lw.r2, m.window)
 
     # ------------------------------------------------------------------ cache
     def _layer_dims(self):
@@ -216,12 +220,12 @@ class MadipelModel:
         out[:, :V] = lg
         return out
 
-    def _attend(self, cache, positions, tables, cu_q=None):
+    def _attend(self, cache, positions, tables, cu_q=None, k_lens=None, max_q=0):
         def run(q, li, out, rows=slice(None)):
             m = self.cfg.layer_specs[li].mixer
             L = self.layers[li]
             res32.window_attn(q[rows], cache.k[li], cache.v[li], positions[rows], tables, L.r1, L.r2, m.window,
-                              out[rows], m.heads, m.kv_heads, cu_q=cu_q)
+                              out[rows], m.heads, m.kv_heads, cu_q=cu_q, k_lens=k_lens, max_q=max_q, bias=L.bias)
         return run
 
     def decode(self, tokens: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor, block_tables: torch.Tensor,
@@ -240,7 +244,8 @@ class MadipelModel:
         both over the paged cache that this step's rows were just written to.  Logits of ``logit_rows``."""
         T = tokens.shape[0]
         dec_run = self._attend(cache, positions, dec["block_tables"]) if n_dec else None
-        chk_run = self._attend(cache, positions, chunk["block_tables"], cu_q=chunk["cu_q"]) if T > n_dec else None
+        chk_run = (self._attend(cache, positions, chunk["block_tables"], cu_q=chunk["cu_q"], k_lens=chunk.get("k_lens"),
+                                max_q=int(chunk.get("max_q", 0))) if T > n_dec else None)
         # (the portion rows' cu_q counts from the first portion row: each part gets its own row slice)
 
         def attend(q, li, out):

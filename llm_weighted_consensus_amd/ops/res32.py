@@ -90,12 +90,27 @@ def residual_add_scaled(x: torch.Tensor, y: torch.Tensor, m: float) -> None:
     kernels().residual_add_scaled(x, y, float(m))
 
 
+def distance_bias(r1: torch.Tensor, r2: torch.Tensor, window: int) -> torch.Tensor:
+    """The table b[h, n] = r1_h ln(1 + r2_h n), n < window (fp32), that the matrix-core kernel reads."""
+    n = torch.arange(window, dtype=torch.float32, device=r1.device)
+    return (r1.float()[:, None] * torch.log1p(r2.float()[:, None] * n[None, :])).contiguous()
+
+
 def window_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, positions: torch.Tensor,
                 block_tables: torch.Tensor, r1: torch.Tensor, r2: torch.Tensor, window: int, out: torch.Tensor,
-                H: int, G: int, cu_q: Optional[torch.Tensor] = None) -> torch.Tensor:
+                H: int, G: int, cu_q: Optional[torch.Tensor] = None, k_lens: Optional[torch.Tensor] = None,
+                max_q: int = 0, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Sliding-window attention over the paged cache with the bias -r1_h ln(1 + r2_h (i - j)); ``q`` fp32
-    [T, H*D] pre-scaled; row t reads table row t (``cu_q`` None) or the item whose ``cu_q`` range holds t."""
-    kernels().window_attn(q, k_cache, v_cache, positions, cu_q, block_tables, r1, r2, int(window), out, int(H), int(G))
+    [T, H*D] pre-scaled; row t reads table row t (``cu_q`` None) or the item whose ``cu_q`` range holds t.
+    Prompt portions over a bf16 cache whose sizes the matrix-core kernel is built for run there (it wants
+    ``k_lens``, ``max_q`` and the ``bias`` table of :func:`distance_bias`); everything else on the general kernel."""
+    K = kernels()
+    if (cu_q is not None and k_lens is not None and bias is not None and max_q > 0 and k_cache.dtype == torch.bfloat16
+            and K.window_attn_mfma_ok(k_cache.shape[2] // G, v_cache.shape[2] // G)):
+        K.window_attn_mfma(q, k_cache, v_cache, positions, cu_q, k_lens, int(max_q), block_tables, bias, int(window), out,
+                           int(H), int(G))
+        return out
+    K.window_attn(q, k_cache, v_cache, positions, cu_q, block_tables, r1, r2, int(window), out, int(H), int(G))
     return out
 
 

@@ -129,6 +129,57 @@ def test_proj_norm_write_and_window_attention(gpu, dtype, tol, H, G, D, Dv, wind
     assert got[:, H * Dv:].abs().max() == 0
 
 
+@pytest.mark.parametrize("H,G,D,Dv,window,bs", [(4, 2, 32, 64, 37, 16), (2, 1, 128, 32, 500, 16), (6, 3, 64, 128, 64, 8),
+                                                 (2, 2, 32, 32, 1, 32)])
+def test_matrix_core_portions(gpu, H, G, D, Dv, window, bs):
+    """Prompt portions on the matrix-core kernel (bf16 cache): several items of unequal length, each the tail of a
+    longer sequence whose head is already cached, tiles cut by item ends, window edges inside and across tiles;
+    against the oracle on the cache's own (bf16) keys and values, and against the general kernel."""
+    from llm_weighted_consensus_amd.models.cache import PagedLayerCache
+    from llm_weighted_consensus_amd.ops import res32
+
+    g = torch.Generator().manual_seed(D + Dv)
+    k_lens, q_lens = [150, 64, 209, 3], [150, 1, 70, 2]
+    nk, nv = G * D, G * Dv
+    nb = sum(-(-n // bs) for n in k_lens) + 2
+    cache = PagedLayerCache([(nk, nv)], nb, bs, "cuda", torch.bfloat16)
+    pages = torch.randperm(nb, generator=g).tolist()
+    temp, r1, r2 = 1 + torch.rand(H, generator=g), 0.3 + torch.rand(H, generator=g), 0.3 + torch.rand(H, generator=g)
+    scale = 0.3
+    width = max(-(-n // bs) for n in k_lens)
+    tables, refs, qs, pos, cu = [], [], [], [], [0]
+    for n, nq_ in zip(k_lens, q_lens):
+        tab = [pages.pop() for _ in range(-(-n // bs))]
+        tables.append(tab + [0] * (width - len(tab)))
+        k = (torch.randn(n, nk, generator=g)).to(torch.bfloat16)
+        v = (torch.randn(n, nv, generator=g)).to(torch.bfloat16)
+        sl = torch.tensor([tab[p // bs] * bs + p % bs for p in range(n)], device=gpu)
+        cache.k[0][sl // bs, sl % bs] = k.to(gpu)
+        cache.v[0][sl // bs, sl % bs] = v.to(gpu)
+        q = torch.randn(n, H * D, generator=g) * 2
+        ref = O.window_attention(q.double().view(n, H, D), k.double().view(n, G, D), v.double().view(n, G, Dv), H, G, window,
+                                 scale, temp.double(), r1.double(), r2.double())
+        refs.append(ref[n - nq_:])
+        qs.append((q.view(n, H, D) * (temp * scale)[None, :, None]).reshape(n, H * D)[n - nq_:])
+        pos.extend(range(n - nq_, n))
+        cu.append(cu[-1] + nq_)
+    ref = torch.cat(refs)
+    qd = torch.cat(qs).float().to(gpu).contiguous()
+    T = qd.shape[0]
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=gpu)
+    r1d, r2d = r1.to(gpu), r2.to(gpu)
+    out_m = torch.zeros(T, H * Dv, dtype=torch.bfloat16, device=gpu)
+    out_g = torch.zeros_like(out_m)
+    assert res32.kernels().window_attn_mfma_ok(D, Dv)
+    res32.window_attn(qd, cache.k[0], cache.v[0], i32(pos), i32(tables), r1d, r2d, window, out_m, H, G, cu_q=i32(cu),
+                      k_lens=i32(k_lens), max_q=max(q_lens), bias=res32.distance_bias(r1d, r2d, window))
+    res32.window_attn(qd, cache.k[0], cache.v[0], i32(pos), i32(tables), r1d, r2d, window, out_g, H, G, cu_q=i32(cu))
+    tol = 0.02  # the outputs are rounded to bf16
+    assert (out_g.cpu().double() - ref).abs().max() < tol
+    assert (out_m.cpu().double() - ref).abs().max() < tol
+    assert (out_m.float() - out_g.float()).abs().max() < tol
+
+
 def test_value_publish_and_plain_modes(gpu):
     from llm_weighted_consensus_amd.ops import res32
 
