@@ -50,12 +50,23 @@ def parse():
     ap.add_argument("--kv-fraction", type=float, default=0.5,
                     help="share of the free device memory the engine's paged KV cache takes")
     ap.add_argument("--profile-steps", action="store_true", help="print a per-phase breakdown")
+    ap.add_argument("--compare-decoders", action="store_true",
+                    help="instead of the headline workload: prefill / decode throughput of the Madipel decoder beside "
+                         "the Llama decoder at equal size (bench_decoders.py), one JSON line per size and design")
+    ap.add_argument("--sizes", default="small,8b-layer", help="--compare-decoders: sizes to run")
+    ap.add_argument("--compare-layers", type=int, default=4, help="--compare-decoders: layers per model")
+    ap.add_argument("--window", type=int, default=0, help="--compare-decoders: Madipel's window (0: the whole context)")
+    ap.add_argument("--designs", default="madipel,llama", help="--compare-decoders: designs to run")
     return ap.parse_args()
 
 
 def main():
     a = parse()
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    if a.compare_decoders:
+        import bench_decoders
+
+        sys.exit(bench_decoders.run(a.sizes, a.compare_layers, prompt_len=2048, window=a.window, designs=a.designs))
     from llm_weighted_consensus_amd.parallel import launch
 
     # `python bench.py --gpus N` without torchrun: this process only launches N ranks (never touches the GPU)

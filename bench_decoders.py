@@ -1,0 +1,117 @@
+#!/usr/bin/env python3
+"""Prefill and decode throughput of two decoder designs at equal size, through the engine.
+
+    python bench.py --compare-decoders [--sizes small,8b-layer] [--compare-layers 4]
+
+For each size a Madipel model (parallel layers, windowed attention with distance bias, xIELU feed-forward, fp32
+residual) and the closest existing decoder (Llama: sequential layers, causal GQA attention with RoPE, SwiGLU) are
+built with random weights at the same width, layer count, head counts, head size, vocabulary and parameter count
+(Madipel's two feed-forward matrices get 1.5x Llama's inner width to match its three), and run through the same
+LLMEngine: prefill = whole prompts in one admission batch (tokens/s), decode = hipGraph decode steps of a fixed
+batch at a fixed context (tokens/s).  One JSON line per (size, design) and a closing summary line.
+"""
+from __future__ import annotations
+
+import json
+import sys
+import time
+
+SIZES = {
+    # name: width, heads, kv_heads, head_dim, llama_ffn, vocab
+    "small": dict(width=2048, heads=16, kv_heads=4, head_dim=128, ffn=8192, vocab=32000),
+    "8b-layer": dict(width=4096, heads=32, kv_heads=8, head_dim=128, ffn=14336, vocab=32000),
+}
+
+
+def _madipel(size: dict, layers: int, window: int, device, seed: int):
+    from llm_weighted_consensus_amd.models.config import MadipelConfig
+    from llm_weighted_consensus_amd.models.madipel import MadipelModel
+
+    layer = {"type": "attention",
+             "mixer": {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["head_dim"], "vdim": size["head_dim"],
+                       "mask": {"size": window}, "scale": size["head_dim"] ** -0.5, "v_mix": True},
+             "mlp": {"kind": "dense", "ff": size["ffn"] * 3 // 2}}
+    cfg = MadipelConfig.from_dict({"architecture": "Madipel", "layers": [layer] * layers, "logit_scale": 1.0,
+                                   "norm": {"eps": 1e-5}, "residual_mult": 0.5, "vocab": size["vocab"],
+                                   "width": size["width"]}, name="madipel-bench")
+    return MadipelModel(cfg, device=device, seed=seed)
+
+
+def _llama(size: dict, layers: int, max_pos: int, device, seed: int):
+    from llm_weighted_consensus_amd.models.config import DecoderConfig
+    from llm_weighted_consensus_amd.models.llama import LlamaModel
+
+    cfg = DecoderConfig("llama-bench", size["vocab"], size["width"], layers, size["heads"], size["kv_heads"],
+                        size["head_dim"], size["ffn"], max_position=max_pos)
+    return LlamaModel(cfg, device=device, seed=seed, max_position=max_pos)
+
+
+def _measure(model, prompt_len: int, n_prompts: int, batch: int, gen: int, reps: int) -> dict:
+    import torch
+
+    from llm_weighted_consensus_amd.engine.engine import LLMEngine
+    from llm_weighted_consensus_amd.engine.sampling import SamplingParams
+    from llm_weighted_consensus_amd.engine.tokenizer import ByteTokenizer
+
+    V = model.cfg.vocab_size
+    bs = 16
+    blocks = (max(n_prompts, batch) + 2) * (-(-(prompt_len + gen + 16) // bs) + 1)
+    eng = LLMEngine(model, ByteTokenizer(V), num_blocks=blocks, max_batch=max(batch, n_prompts),
+                    max_model_len=prompt_len + gen + 16, prefill_token_budget=n_prompts * prompt_len, prefix_sharing=False,
+                    kv_reserve_tokens=None)
+    g = torch.Generator().manual_seed(7)
+
+    def prompts(n):
+        return [torch.randint(0, 255, (prompt_len,), generator=g).tolist() for _ in range(n)]
+
+    def run(n, new):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.generate(prompts(n), SamplingParams(temperature=0.0, max_tokens=new, ignore_eos=True))
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    run(n_prompts, 1)          # warm-up: kernels, library heuristics
+    run(batch, gen)            # warm-up: the decode bucket's tuning and graph capture
+    t_pre = min(run(n_prompts, 1) for _ in range(reps))
+    t_one = min(run(batch, 1) for _ in range(reps))
+    t_gen = min(run(batch, gen) for _ in range(reps))
+    del eng
+    torch.cuda.empty_cache()
+    return {"prefill_tok_s": n_prompts * prompt_len / t_pre, "prefill_ms": t_pre * 1e3,
+            "decode_tok_s": batch * (gen - 1) / max(t_gen - t_one, 1e-9), "decode_ms_per_step": (t_gen - t_one) / (gen - 1) * 1e3}
+
+
+def run(sizes: str = "small,8b-layer", layers: int = 4, prompt_len: int = 2048, n_prompts: int = 8, batch: int = 64,
+        gen: int = 33, window: int = 0, reps: int = 2, designs: str = "madipel,llama") -> int:
+    import torch
+
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    window = window or (prompt_len + gen + 16)  # default: the window covers the context (equal attention work)
+    summary = {}
+    for name in sizes.split(","):
+        size = SIZES[name]
+        for design in designs.split(","):
+            model = (_madipel(size, layers, window, dev, 3) if design == "madipel"
+                     else _llama(size, layers, prompt_len + gen + 80, dev, 3))
+            r = _measure(model, prompt_len, n_prompts, batch, gen, reps)
+            params = model.cfg.params()
+            del model
+            torch.cuda.empty_cache()
+            line = {"bench": "compare-decoders", "size": name, "design": design, "layers": layers, "params": params,
+                    "prompt_len": prompt_len, "prompts": n_prompts, "decode_batch": batch, "window": window if design == "madipel" else None,
+                    **{k: round(v, 3) for k, v in r.items()}, "dtype": "bf16", "data": "synthetic"}
+            print(json.dumps(line), flush=True)
+            summary.setdefault(name, {})[design] = r
+    out = {}
+    for name, d in summary.items():
+        if "madipel" in d and "llama" in d:
+            out[name] = {"prefill_ratio": round(d["madipel"]["prefill_tok_s"] / d["llama"]["prefill_tok_s"], 3),
+                         "decode_ratio": round(d["madipel"]["decode_tok_s"] / d["llama"]["decode_tok_s"], 3)}
+    print(json.dumps({"bench": "compare-decoders", "madipel_over_llama": out}), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(run())

@@ -20,6 +20,9 @@ int r32_window_attn_mfma_ok(int, int);
 int r32_window_attn_mfma(const float*, const void*, const void*, long long, long long, int, const int*, const int*,
                          const int*, int, int, const int*, int, const float*, int, void*, int, int, int, int, int,
                          hipStream_t);
+int r32_window_attn_decode_splits(int, int, int, int);
+int r32_window_attn_decode(const float*, const void*, const void*, long long, long long, int, const int*, const int*, int,
+                           const float*, int, float*, float*, int, int, void*, int, int, int, int, int, int, hipStream_t);
 }
 
 namespace {
@@ -39,6 +42,14 @@ void want(const Tensor& t, torch::ScalarType st, const char* name) {
 }
 
 void done(int rc, const char* name) { TORCH_CHECK(rc == 0, name, ": launch failed (", rc, ")"); }
+
+// One layer's views of the paged pool: K [NB, BS, nk] token rows, V [NB, BS/4, nv, 4] 4-token interleaved.
+void cache_layout(const Tensor& k, const Tensor& v, int& NB, int& BS, int& nk, int& nv, const char* name) {
+  TORCH_CHECK(k.dim() == 3 && v.dim() == 4 && v.size(3) == 4, name, ": K [NB, BS, nk] and V [NB, BS/4, nv, 4] expected");
+  NB = (int)k.size(0), BS = (int)k.size(1), nk = (int)k.size(2), nv = (int)v.size(2);
+  TORCH_CHECK(BS % 4 == 0 && v.size(0) == NB && v.size(1) == BS / 4 && k.stride(2) == 1 && k.stride(1) == nk &&
+                  v.stride(3) == 1 && v.stride(2) == 4 && v.stride(1) == 4 * (int64_t)nv, name, ": cache layout");
+}
 
 // rows of a 2-d tensor whose last dimension is dense; returns the leading dimension in elements
 int row_stride(const Tensor& t, const char* name) {
@@ -90,12 +101,10 @@ void proj_norm_kv_write(Tensor proj, Tensor wq, Tensor wk, Tensor head_scale, c1
   want(slots, torch::kInt32, "proj_norm_kv_write slots");
   want(q_out, torch::kFloat32, "proj_norm_kv_write q_out");
   want(head_scale, torch::kFloat32, "proj_norm_kv_write head_scale");
-  TORCH_CHECK(k_cache.dim() == 3 && v_cache.dim() == 3 && k_cache.is_cuda() && v_cache.is_cuda() &&
-                  k_cache.scalar_type() == proj.scalar_type() && v_cache.scalar_type() == proj.scalar_type(),
-              "proj_norm_kv_write: caches [NB, BS, n] of the activation dtype");
-  const int NB = (int)k_cache.size(0), BS = (int)k_cache.size(1), nk = (int)k_cache.size(2), nv = (int)v_cache.size(2);
-  TORCH_CHECK(v_cache.size(0) == NB && v_cache.size(1) == BS && k_cache.stride(2) == 1 && k_cache.stride(1) == nk &&
-                  v_cache.stride(2) == 1 && v_cache.stride(1) == nv, "proj_norm_kv_write: cache layout");
+  TORCH_CHECK(k_cache.is_cuda() && v_cache.is_cuda() && k_cache.scalar_type() == proj.scalar_type() &&
+                  v_cache.scalar_type() == proj.scalar_type(), "proj_norm_kv_write: caches of the activation dtype");
+  int NB, BS, nk, nv;
+  cache_layout(k_cache, v_cache, NB, BS, nk, nv, "proj_norm_kv_write");
   const int nq = (int)(H * D);
   TORCH_CHECK(H > 0 && D > 0 && proj.size(1) >= nq + nk + nv && slots.numel() == T && q_out.numel() == (int64_t)T * nq &&
                   wq.numel() == nq && wk.numel() == nk && head_scale.numel() == H && wq.scalar_type() == proj.scalar_type() &&
@@ -148,15 +157,14 @@ void window_attn(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, c10
   want(block_tables, torch::kInt32, "window_attn block_tables");
   want(r1, torch::kFloat32, "window_attn r1");
   want(r2, torch::kFloat32, "window_attn r2");
-  TORCH_CHECK(k_cache.dim() == 3 && v_cache.dim() == 3 && v_cache.is_cuda() && v_cache.scalar_type() == k_cache.scalar_type() &&
-                  out.is_cuda() && out.scalar_type() == k_cache.scalar_type(), "window_attn: caches and out share a dtype");
+  TORCH_CHECK(v_cache.is_cuda() && v_cache.scalar_type() == k_cache.scalar_type() && out.is_cuda() &&
+                  out.scalar_type() == k_cache.scalar_type(), "window_attn: caches and out share a dtype");
   const int T = (int)positions.numel();
-  const int NB = (int)k_cache.size(0), BS = (int)k_cache.size(1), nk = (int)k_cache.size(2), nv = (int)v_cache.size(2);
+  int NB, BS, nk, nv;
+  cache_layout(k_cache, v_cache, NB, BS, nk, nv, "window_attn");
   TORCH_CHECK(G > 0 && H > 0 && H % G == 0 && nk % G == 0 && nv % G == 0, "window_attn: head counts");
   const int D = nk / (int)G, Dv = nv / (int)G;
   const int ldo = row_stride(out, "window_attn out");
-  TORCH_CHECK(v_cache.size(0) == NB && v_cache.size(1) == BS && k_cache.stride(2) == 1 && k_cache.stride(1) == nk &&
-                  v_cache.stride(2) == 1 && v_cache.stride(1) == nv, "window_attn: cache layout");
   TORCH_CHECK(q.numel() == (int64_t)T * H * D && out.size(0) == T && out.size(1) == H * Dv && r1.numel() == H &&
                   r2.numel() == H && window >= 1 && block_tables.dim() == 2, "window_attn: shapes disagree");
   const int items = (int)block_tables.size(0), width = (int)block_tables.size(1);
@@ -187,19 +195,18 @@ void window_attn_mfma(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions
   want(cu_q, torch::kInt32, "window_attn_mfma cu_q");
   want(k_lens, torch::kInt32, "window_attn_mfma k_lens");
   want(bias, torch::kFloat32, "window_attn_mfma bias");
-  TORCH_CHECK(k_cache.dim() == 3 && v_cache.dim() == 3 && k_cache.is_cuda() && v_cache.is_cuda() && out.is_cuda() &&
-                  k_cache.scalar_type() == torch::kBFloat16 && v_cache.scalar_type() == torch::kBFloat16 &&
-                  out.scalar_type() == torch::kBFloat16, "window_attn_mfma: bf16 caches and out");
+  TORCH_CHECK(k_cache.is_cuda() && v_cache.is_cuda() && out.is_cuda() && k_cache.scalar_type() == torch::kBFloat16 &&
+                  v_cache.scalar_type() == torch::kBFloat16 && out.scalar_type() == torch::kBFloat16,
+              "window_attn_mfma: bf16 caches and out");
   const int T = (int)positions.numel();
-  const int NB = (int)k_cache.size(0), BS = (int)k_cache.size(1), nk = (int)k_cache.size(2), nv = (int)v_cache.size(2);
+  int NB, BS, nk, nv;
+  cache_layout(k_cache, v_cache, NB, BS, nk, nv, "window_attn_mfma");
   TORCH_CHECK(G > 0 && H > 0 && H % G == 0 && nk % G == 0 && nv % G == 0, "window_attn_mfma: head counts");
   const int D = nk / (int)G, Dv = nv / (int)G;
   TORCH_CHECK(r32_window_attn_mfma_ok(D, Dv), "window_attn_mfma: sizes not built");
   const int ldo = row_stride(out, "window_attn_mfma out");
-  TORCH_CHECK(v_cache.size(0) == NB && v_cache.size(1) == BS && k_cache.stride(2) == 1 && k_cache.stride(1) == nk &&
-                  v_cache.stride(2) == 1 && v_cache.stride(1) == nv && k_cache.stride(0) % 8 == 0 && v_cache.stride(0) % 8 == 0 &&
-                  ((uintptr_t)k_cache.data_ptr() & 15) == 0 && ((uintptr_t)v_cache.data_ptr() & 15) == 0,
-              "window_attn_mfma: cache layout");
+  TORCH_CHECK(k_cache.stride(0) % 8 == 0 && v_cache.stride(0) % 8 == 0 && ((uintptr_t)k_cache.data_ptr() & 15) == 0 &&
+                  ((uintptr_t)v_cache.data_ptr() & 15) == 0, "window_attn_mfma: cache alignment");
   const int items = (int)block_tables.size(0);
   TORCH_CHECK(block_tables.dim() == 2 && cu_q.numel() == items + 1 && k_lens.numel() == items && max_q >= 1 &&
                   q.numel() == (int64_t)T * H * D && out.size(0) == T && out.size(1) == H * Dv && window >= 1 &&
@@ -209,6 +216,38 @@ void window_attn_mfma(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions
                             k_lens.data_ptr<int>(), items, (int)max_q, block_tables.data_ptr<int>(),
                             (int)block_tables.size(1), bias.data_ptr<float>(), (int)window, out.data_ptr(), ldo, (int)H, (int)G,
                             D, Dv, stream()), "window_attn_mfma");
+}
+
+// One new token per sequence on the matrix cores (bf16 caches): row b reads table row b, its key range ends at
+// positions[b].  max_keys: a host-side upper bound of the keys a row sees (min(window, longest context)).
+void window_attn_decode(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, Tensor block_tables, Tensor bias,
+                        int64_t window, int64_t max_keys, Tensor out, int64_t H, int64_t G) {
+  want(q, torch::kFloat32, "window_attn_decode q");
+  want(positions, torch::kInt32, "window_attn_decode positions");
+  want(block_tables, torch::kInt32, "window_attn_decode block_tables");
+  want(bias, torch::kFloat32, "window_attn_decode bias");
+  TORCH_CHECK(k_cache.is_cuda() && v_cache.is_cuda() && out.is_cuda() && k_cache.scalar_type() == torch::kBFloat16 &&
+                  v_cache.scalar_type() == torch::kBFloat16 && out.scalar_type() == torch::kBFloat16,
+              "window_attn_decode: bf16 caches and out");
+  const int B = (int)positions.numel();
+  int NB, BS, nk, nv;
+  cache_layout(k_cache, v_cache, NB, BS, nk, nv, "window_attn_decode");
+  TORCH_CHECK(G > 0 && H > 0 && H % G == 0 && nk % G == 0 && nv % G == 0, "window_attn_decode: head counts");
+  const int D = nk / (int)G, Dv = nv / (int)G;
+  TORCH_CHECK(r32_window_attn_mfma_ok(D, Dv), "window_attn_decode: sizes not built");
+  const int ldo = row_stride(out, "window_attn_decode out");
+  TORCH_CHECK(k_cache.stride(0) % 8 == 0 && v_cache.stride(0) % 8 == 0 && ((uintptr_t)k_cache.data_ptr() & 15) == 0 &&
+                  ((uintptr_t)v_cache.data_ptr() & 15) == 0, "window_attn_decode: cache alignment");
+  TORCH_CHECK(block_tables.dim() == 2 && block_tables.size(0) >= B && q.numel() == (int64_t)B * H * D && out.size(0) == B &&
+                  out.size(1) == H * Dv && window >= 1 && max_keys >= 1 && bias.numel() == H * window,
+              "window_attn_decode: shapes disagree");
+  const int S = r32_window_attn_decode_splits(B, (int)G, (int)(H / G), (int)max_keys);
+  auto part = torch::empty({(int64_t)B * H * S * (Dv + 2)}, q.options());
+  float* po = part.data_ptr<float>();
+  done(r32_window_attn_decode(q.data_ptr<float>(), k_cache.data_ptr(), v_cache.data_ptr(), (long long)k_cache.stride(0),
+                              (long long)v_cache.stride(0), BS, positions.data_ptr<int>(), block_tables.data_ptr<int>(),
+                              (int)block_tables.size(1), bias.data_ptr<float>(), (int)window, po, po + (int64_t)B * H * S * Dv, S,
+                              (int)max_keys, out.data_ptr(), ldo, B, (int)H, (int)G, D, Dv, stream()), "window_attn_decode");
 }
 
 }  // namespace
@@ -223,4 +262,5 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("window_attn", &window_attn);
   m.def("window_attn_mfma", &window_attn_mfma);
   m.def("window_attn_mfma_ok", &window_attn_mfma_ok);
+  m.def("window_attn_decode", &window_attn_decode);
 }

@@ -7,7 +7,7 @@
 //   layernorm_f32       (x - mean) / sqrt(var + eps) * w + b over fp32 rows (optionally gathered rows)
 //   proj_norm_kv_write  the q and k projections RMS-normalised over the WHOLE projection (all heads at once),
 //                       q scaled per head (softmax scale x temperature) into an fp32 buffer, k into the paged
-//                       cache; v blended with the values of an earlier layer (v <- (1 - lam) v + lam v0) or
+//                       cache; v (4-token interleaved in its pages) blended with the values of an earlier layer (v <- (1 - lam) v + lam v0) or
 //                       published as that v0, then into the paged cache
 //   xielu               z > 0: ap z^2 + z/2;  z <= 0: an (expm1(z) - z) + z/2, ap = softplus(p), an = 1/2 + softplus(q)
 //   residual_add_scaled x += m * y
@@ -106,12 +106,13 @@ __global__ void proj_norm_kv_write_kernel(const AT* __restrict__ proj, int ldp, 
       Elem<AT>::st(kc + i, Elem<AT>::ld(pr + nq + i) * rk * Elem<AT>::ld(wk + i));
   }
   const float lam = vmode == 2 ? Elem<AT>::ld(lam_p) : 0.f;
-  AT* vc = v_cache + blk * vb_stride + off * nv;
+  // V is 4-token interleaved: [block][offset / 4][column][offset % 4]
+  AT* vc = v_cache + blk * vb_stride + (off >> 2) * (4LL * nv) + (off & 3);
   for (int i = threadIdx.x; i < nv; i += blockDim.x) {
     float v = Elem<AT>::ld(pr + nq + nk + i);
     if (vmode == 1) v0[(size_t)t * nv + i] = v;
     if (vmode == 2) v = (1.0f - lam) * v + lam * v0[(size_t)t * nv + i];
-    if (write) Elem<AT>::st(vc + i, v);
+    if (write) Elem<AT>::st(vc + 4 * i, v);
   }
 }
 

@@ -1,8 +1,9 @@
 """Paged K/V cache for decoders whose layers differ (key size != value size, other head counts per layer).
 
 One pool ``[num_blocks, block_elems]`` holds, per block, every layer's keys then values for ``block_size`` tokens;
-a layer's K is the strided view ``[num_blocks, block_size, G*D]`` and its V ``[num_blocks, block_size, G*Dv]``
-(token-major rows, the layout of ``csrc/kernels/res32/wattn.hip``).  Block ids come from the engine's C++ block
+a layer's K is the strided view ``[num_blocks, block_size, G*D]`` (token-major rows) and its V the 4-token
+interleaved view ``[num_blocks, block_size/4, G*Dv, 4]`` — four consecutive tokens of one value column are one
+8-byte word, the matrix cores' operand for the weighted sum without a transpose (``csrc/kernels/res32/wattn.hip``).  Block ids come from the engine's C++ block
 manager like every other model's; whole blocks are copied (copy-on-write forks), exported and imported (swap,
 prefill hand-over) with one index operation on the pool."""
 from __future__ import annotations
@@ -17,6 +18,8 @@ class PagedLayerCache:
                  dtype=torch.bfloat16):
         """``layer_dims``: per layer (G*D, G*Dv), the key and value row sizes."""
         self.num_blocks, self.block_size, self.dtype = int(num_blocks), int(block_size), dtype
+        if block_size % 4:
+            raise ValueError("PagedLayerCache: block_size must be a multiple of 4 (4-token interleaved values)")
         self.layer_dims = [(int(a), int(b)) for a, b in layer_dims]
         offs, o = [], 0
         for nk, nv in self.layer_dims:
@@ -31,11 +34,22 @@ class PagedLayerCache:
         self.v: List[torch.Tensor] = []
         for (nk, nv), (ko, vo) in zip(self.layer_dims, offs):
             self.k.append(self.pool[:, ko:ko + block_size * nk].view(self.num_blocks, block_size, nk))
-            self.v.append(self.pool[:, vo:vo + block_size * nv].view(self.num_blocks, block_size, nv))
+            self.v.append(self.pool[:, vo:vo + block_size * nv].view(self.num_blocks, block_size // 4, nv, 4))
 
     @staticmethod
     def elems_per_block(layer_dims: Sequence[Tuple[int, int]], block_size: int) -> int:
         return sum(-(-block_size * nk // 8) * 8 + -(-block_size * nv // 8) * 8 for nk, nv in layer_dims)
+
+    # token rows by cache slot (slot = block * block_size + offset): tools and tests, not the product path
+    def rows(self, layer: int, slots: torch.Tensor):
+        """(K rows [n, G*D], V rows [n, G*Dv]) of the tokens at ``slots`` (int64)."""
+        b, o = slots // self.block_size, slots % self.block_size
+        return self.k[layer][b, o], self.v[layer][b, o // 4, :, o % 4]
+
+    def set_rows(self, layer: int, slots: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> None:
+        b, o = slots // self.block_size, slots % self.block_size
+        self.k[layer][b, o] = k.to(self.pool.dtype)
+        self.v[layer][b, o // 4, :, o % 4] = v.to(self.pool.dtype)
 
     def copy_blocks(self, pairs: torch.Tensor) -> None:
         """(src, dst) block copies queued by the block manager's copy-on-write."""

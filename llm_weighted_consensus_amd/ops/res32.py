@@ -6,7 +6,7 @@ while the activations between kernels are bf16 (serving) or fp32 (exact mode).  
 missing (a fresh checkout), and there is no eager-PyTorch fallback.
 
 Cache layout shared with :class:`..models.cache.PagedLayerCache`: per layer K ``[num_blocks, block_size, G*D]``
-and V ``[num_blocks, block_size, G*Dv]`` as strided views of one pool.
+and V ``[num_blocks, block_size/4, G*Dv, 4]`` (4-token interleaved) as strided views of one pool.
 """
 from __future__ import annotations
 
@@ -102,9 +102,15 @@ def window_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, p
                 max_q: int = 0, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Sliding-window attention over the paged cache with the bias -r1_h ln(1 + r2_h (i - j)); ``q`` fp32
     [T, H*D] pre-scaled; row t reads table row t (``cu_q`` None) or the item whose ``cu_q`` range holds t.
-    Prompt portions over a bf16 cache whose sizes the matrix-core kernel is built for run there (it wants
-    ``k_lens``, ``max_q`` and the ``bias`` table of :func:`distance_bias`); everything else on the general kernel."""
+    Over a bf16 cache whose sizes the matrix-core kernels are built for, prompt portions run on the portion kernel
+    (it wants ``k_lens``, ``max_q`` and the ``bias`` table of :func:`distance_bias`) and decode rows on the
+    split-key decode kernel (``bias``); everything else on the general kernel."""
     K = kernels()
+    if (cu_q is None and bias is not None and k_cache.dtype == torch.bfloat16 and positions.numel() > 0
+            and K.window_attn_mfma_ok(k_cache.shape[2] // G, v_cache.shape[2] // G)):
+        max_keys = min(int(window), block_tables.shape[1] * k_cache.shape[1])
+        K.window_attn_decode(q, k_cache, v_cache, positions, block_tables, bias, int(window), max_keys, out, int(H), int(G))
+        return out
     if (cu_q is not None and k_lens is not None and bias is not None and max_q > 0 and k_cache.dtype == torch.bfloat16
             and K.window_attn_mfma_ok(k_cache.shape[2] // G, v_cache.shape[2] // G)):
         K.window_attn_mfma(q, k_cache, v_cache, positions, cu_q, k_lens, int(max_q), block_tables, bias, int(window), out,

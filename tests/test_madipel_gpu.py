@@ -113,8 +113,7 @@ def test_proj_norm_write_and_window_attention(gpu, dtype, tol, H, G, D, Dv, wind
     q_dev = res32.proj_norm_kv_write(_dev(proj, dtype), _dev(wq, dtype), _dev(wk, dtype), head_scale,
                                      torch.tensor(slots, dtype=torch.int32, device=gpu), cache.k[0], cache.v[0], H, D, eps,
                                      lam=_dev(lam, dtype), v0=v_first.to(gpu), vmode=2)
-    kc = cache.k[0].reshape(-1, nk)[torch.tensor(slots, device=gpu)].cpu().double()
-    vc = cache.v[0].reshape(-1, nv)[torch.tensor(slots, device=gpu)].cpu().double()
+    kc, vc = (t.cpu().double() for t in cache.rows(0, torch.tensor(slots, device=gpu)))
     assert (kc - k).abs().max() < tol and (vc - v).abs().max() < tol * 3
     pos = torch.arange(n, dtype=torch.int32, device=gpu)
     out = torch.zeros(n, H * Dv + 3, dtype=dtype, device=gpu)
@@ -154,8 +153,7 @@ def test_matrix_core_portions(gpu, H, G, D, Dv, window, bs):
         k = (torch.randn(n, nk, generator=g)).to(torch.bfloat16)
         v = (torch.randn(n, nv, generator=g)).to(torch.bfloat16)
         sl = torch.tensor([tab[p // bs] * bs + p % bs for p in range(n)], device=gpu)
-        cache.k[0][sl // bs, sl % bs] = k.to(gpu)
-        cache.v[0][sl // bs, sl % bs] = v.to(gpu)
+        cache.set_rows(0, sl, k.to(gpu), v.to(gpu))
         q = torch.randn(n, H * D, generator=g) * 2
         ref = O.window_attention(q.double().view(n, H, D), k.double().view(n, G, D), v.double().view(n, G, Dv), H, G, window,
                                  scale, temp.double(), r1.double(), r2.double())
@@ -178,6 +176,12 @@ def test_matrix_core_portions(gpu, H, G, D, Dv, window, bs):
     assert (out_g.cpu().double() - ref).abs().max() < tol
     assert (out_m.cpu().double() - ref).abs().max() < tol
     assert (out_m.float() - out_g.float()).abs().max() < tol
+    # the last token of every item as a decode row (split over the keys when the window is long)
+    last = [c - 1 for c in cu[1:]]
+    out_d = torch.zeros(len(last), H * Dv, dtype=torch.bfloat16, device=gpu)
+    res32.window_attn(qd[last].contiguous(), cache.k[0], cache.v[0], i32([pos[r] for r in last]), i32(tables), r1d, r2d,
+                      window, out_d, H, G, bias=res32.distance_bias(r1d, r2d, window))
+    assert (out_d.cpu().double() - ref[last]).abs().max() < tol
 
 
 def test_value_publish_and_plain_modes(gpu):
@@ -195,11 +199,11 @@ def test_value_publish_and_plain_modes(gpu):
                              torch.tensor(slots, dtype=torch.int32, device=gpu), cache.k[0], cache.v[0], H, D, 1e-6, v0=v0, vmode=1)
     assert torch.equal(v0.cpu(), proj[:, H * D + nk:])
     rows = [s for s in slots if s >= 0]
-    vc = cache.v[0].reshape(-1, nv)[torch.tensor(rows, device=gpu)].cpu()
-    assert torch.equal(vc, proj[[0, 1, 3, 4, 5], H * D + nk:])
-    untouched = torch.ones(cache.num_blocks * 4, dtype=torch.bool)
-    untouched[rows] = False
-    assert torch.equal(cache.k[0].reshape(-1, nk).cpu()[untouched], before[:, :4 * nk].reshape(-1, nk).cpu()[untouched])
+    kc, vc = cache.rows(0, torch.tensor(rows, device=gpu))
+    assert torch.equal(vc.cpu(), proj[[0, 1, 3, 4, 5], H * D + nk:])
+    rest = torch.tensor([s for s in range(cache.num_blocks * 4) if s not in rows], device=gpu)
+    for a, b in zip(cache.rows(0, rest), (before[:, :4 * nk].reshape(-1, nk)[rest], torch.zeros(len(rest), nv, device=gpu))):
+        assert torch.equal(a, b)
 
 
 @pytest.mark.parametrize("decode", [False, True])
@@ -219,8 +223,7 @@ def test_window_edge_and_far_key_stand_out(gpu, decode):
     v[special] = torch.tensor([0.0, 7.0, 0.0, 0.0])
     cache, table, slots = _paged(n, bs, D, Dv, torch.float32, perm_seed=3)
     sl = torch.tensor(slots, device=gpu)
-    cache.k[0][sl // bs, sl % bs] = k.to(gpu)  # (the layer views are strided: index them, a reshape would copy)
-    cache.v[0][sl // bs, sl % bs] = v.to(gpu)
+    cache.set_rows(0, sl, k.to(gpu), v.to(gpu))
     rows = [special, special + 1, special + window - 1, special + window, n - 1]
     q = torch.zeros(len(rows), D, device=gpu)
     q[:, 1] = 1.0
@@ -249,6 +252,11 @@ CONFIGS = {
         dict(heads=4, kv_heads=2, dim=16, vdim=8, window=6, v_mix=True, ff=None),
         dict(heads=2, kv_heads=1, dim=8, vdim=16, window=19, v_mix=True, ff=40),
         dict(heads=8, kv_heads=4, dim=4, vdim=4, window=3, v_mix=True, ff=72)]),
+    # sizes the matrix-core kernels take (bf16): dim != vdim, one window shorter than a key tile, one longer
+    "cores": dict(width=64, vocab=320, layers=[
+        dict(heads=4, kv_heads=2, dim=32, vdim=64, window=40, v_mix=True, ff=64),
+        dict(heads=2, kv_heads=1, dim=128, vdim=32, window=7, v_mix=False, ff=None),
+        dict(heads=4, kv_heads=2, dim=32, vdim=64, window=90, v_mix=True, ff=48)]),
     # odd sizes, heads == kv_heads, a window longer than any test prompt and a window of one
     "odd": dict(width=40, vocab=97, layers=[
         dict(heads=3, kv_heads=3, dim=12, vdim=20, window=1000, v_mix=True, ff=50),
@@ -305,32 +313,33 @@ def test_whole_prompt_and_layers(gpu, tmp_path, name, dtype):
     assert eng.bm.num_free == eng.bm.num_blocks
 
 
-@pytest.mark.parametrize("name", list(CONFIGS))
-def test_decode_token_by_token_and_portions(gpu, tmp_path, name):
+@pytest.mark.parametrize("name,dtype", [("mixed", torch.float32), ("odd", torch.float32), ("cores", torch.float32),
+                                        ("cores", torch.bfloat16)])
+def test_decode_token_by_token_and_portions(gpu, tmp_path, name, dtype):
     """The same logits whether a prompt comes whole, token by token from the first token on, or in portions of
     changing sizes (down to two tokens, cut inside pages and windows)."""
-    cfg, W, model, eng = _build(tmp_path, name, torch.float32)
+    cfg, W, model, eng = _build(tmp_path, name, dtype)
     toks = _tokens(75, cfg["vocab"], 2)
     ref = O.forward(cfg, W, toks)
     rows = []
     for i, t in enumerate(toks):
         rows.append(eng.step_tokens([("d", [t], [0])], ["d"] if i + 1 == len(toks) else []))
-    assert _err(torch.cat(rows), ref) < TOL[torch.float32]
+    assert _err(torch.cat(rows), ref) < TOL[dtype]
     for sizes in ([2, 2, 13, 3, 16, 2, 30, 7], [17, 16, 15, 2, 25], [1, 2, 5, 67]):
         assert sum(sizes) == len(toks)
         rows, a = [], 0
         for n in sizes:
             rows.append(eng.step_tokens([("p", toks[a:a + n], list(range(n)))], ["p"] if a + n == len(toks) else []))
             a += n
-        assert _err(torch.cat(rows), ref) < TOL[torch.float32]
+        assert _err(torch.cat(rows), ref) < TOL[dtype]
     assert eng.bm.num_free == eng.bm.num_blocks
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_unequal_batches_and_page_reuse(gpu, tmp_path, dtype):
+@pytest.mark.parametrize("name,dtype", [("mixed", torch.float32), ("mixed", torch.bfloat16), ("cores", torch.bfloat16)])
+def test_unequal_batches_and_page_reuse(gpu, tmp_path, name, dtype):
     """Up to four live sequences of unequal lengths, portions beside single tokens, in a pool so small that pages
     are freed and taken again; every position equals the sequence run alone."""
-    cfg, W, model, eng = _build(tmp_path, "mixed", dtype, num_blocks=14)
+    cfg, W, model, eng = _build(tmp_path, name, dtype, num_blocks=14)
     seqs = {k: _tokens(n, cfg["vocab"], 10 + i) for i, (k, n) in enumerate([("a", 70), ("b", 9), ("c", 40), ("d", 33), ("e", 58), ("f", 1)])}
     ref = {k: O.forward(cfg, W, t) for k, t in seqs.items()}
     at = {k: 0 for k in seqs}
