@@ -130,6 +130,25 @@ __global__ void xielu_kernel(const AT* __restrict__ in, int ldi, const AT* __res
   }
 }
 
+// bf16 rows whose width, leading dimensions and bases are multiples of 8 elements: 16 bytes per lane
+__global__ void xielu_bf16x8_kernel(const bf16_t* __restrict__ in, int ldi, const bf16_t* __restrict__ pq,
+                                    bf16_t* __restrict__ out, int ldo, int n8, long long total8) {
+  const float ap = softplus(bf2f(pq[0])), an = 0.5f + softplus(bf2f(pq[1]));
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < total8;
+       e += (long long)gridDim.x * blockDim.x) {
+    const long long r = e / n8;
+    const int c = (int)(e - r * n8) * 8;
+    float f[8];
+    unpack8(*reinterpret_cast<const uint4v*>(in + r * ldi + c), f);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float z = f[k];
+      f[k] = z > 0.f ? ap * z * z + 0.5f * z : an * (expm1f(z) - z) + 0.5f * z;
+    }
+    *reinterpret_cast<uint4v*>(out + r * ldo + c) = pack8(f);
+  }
+}
+
 template <typename AT>
 __global__ void residual_add_scaled_kernel(float* __restrict__ x, const AT* __restrict__ y, float m, long long total) {
   for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < total;
@@ -190,6 +209,11 @@ int r32_proj_norm_kv_write(const void* proj, int ldp, const void* wq, const void
 int r32_xielu(const void* in, int ldi, const void* pq, void* out, int ldo, int T, int n, int f32, hipStream_t s) {
   const long long total = (long long)T * n;
   if (total <= 0) return 0;
+  if (!f32 && n % 8 == 0 && ldi % 8 == 0 && ldo % 8 == 0 && ((uintptr_t)in & 15) == 0 && ((uintptr_t)out & 15) == 0) {
+    xielu_bf16x8_kernel<<<grid_for(total / 8, 256), 256, 0, s>>>((const bf16_t*)in, ldi, (const bf16_t*)pq, (bf16_t*)out, ldo,
+                                                                 n / 8, total / 8);
+    return (int)hipGetLastError();
+  }
   const int g = grid_for(total, 256);
   R32_DISPATCH(f32,
                (xielu_kernel<bf16_t><<<g, 256, 0, s>>>((const bf16_t*)in, ldi, (const bf16_t*)pq, (bf16_t*)out, ldo, n, total)),

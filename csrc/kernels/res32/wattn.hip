@@ -213,8 +213,10 @@ constexpr int kVPad = 40;  // keys per V^T row in LDS (32 + 8: rows stay 16-byte
 template <int ND, int NV>
 __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaParams p) {
   constexpr int D = 32 * ND, DV = 16 * NV, KLD = D + 8;
+  constexpr int KCH = (32 * (D / 8) + 255) / 256, VCH = (8 * (DV / 2) + 255) / 256;  // 16-byte words per thread and tile
   __shared__ __attribute__((aligned(16))) bf16_t K_s[32 * KLD];
   __shared__ __attribute__((aligned(16))) bf16_t Vt_s[DV * kVPad];
+  __shared__ float bias_s[96];  // the tile's bias by (row - key + 31): rows 0..63 of the workgroup, keys 0..31 of the tile
   const int it = blockIdx.x / p.tiles_per_item, tile = blockIdx.x % p.tiles_per_item;
   const int q_begin = p.cu_q[it], q_end = p.cu_q[it + 1];
   const int row0 = q_begin + tile * 64;
@@ -222,15 +224,16 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
   const int h = blockIdx.y, H = p.H, g = h / (H / p.G), G = p.G;
   const int nrows = min(64, q_end - row0);
   const int k_len = p.k_lens[it];
-  const int pos0 = p.positions[row0], pos_last = p.positions[row0 + nrows - 1];
+  const int pos0 = p.positions[row0], pos_last = pos0 + nrows - 1;  // positions ascend by one along the rows
   const int j_lo = max(0, pos0 - p.window + 1), j_hi = min(pos_last, k_len - 1);
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, r16 = lane & 15, g4 = lane >> 4;
   const int* table = p.block_tables + (size_t)it * p.bt_width;
   const int BS = p.block_size;
+  typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
 
   const int qrow = 16 * w + r16;
   const bool q_valid = qrow < nrows;
-  const int i_q = q_valid ? p.positions[row0 + qrow] : -1;
+  const int i_q = pos0 + qrow;
   short8 qhi[ND], qlo[ND];
 #pragma unroll
   for (int kd = 0; kd < ND; ++kd) {
@@ -252,33 +255,64 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
   float m = -1e30f, l = 0.f;
   const float* bias_h = p.bias + (size_t)h * p.window;
 
-  for (int kt = j_lo / 32; kt <= j_hi / 32; ++kt) {
-    __syncthreads();
-    for (int c = tid; c < 32 * (D / 8); c += 256) {
+  // a tile's words are fetched into registers one tile ahead (the loads fly while the previous tile is computed)
+  uint4v kreg[KCH], vreg[VCH];
+  float breg = 0.f;
+  auto fetch = [&](int kt) {
+#pragma unroll
+    for (int u = 0; u < KCH; ++u) {
+      const int c = tid + 256 * u;
       const int key = c / (D / 8), dc = c % (D / 8);
       const int j = kt * 32 + key;
-      uint4v val = uint4v{0u, 0u, 0u, 0u};
-      if (j <= j_hi) {
+      kreg[u] = uint4v{0u, 0u, 0u, 0u};
+      if (c < 32 * (D / 8) && j <= j_hi) {
         const long long page = table[j / BS];
-        val = *reinterpret_cast<const uint4v*>(p.k_cache + page * p.kb_stride + ((long long)(j % BS) * G + g) * D + dc * 8);
+        kreg[u] = *reinterpret_cast<const uint4v*>(p.k_cache + page * p.kb_stride + ((long long)(j % BS) * G + g) * D + dc * 8);
       }
-      *reinterpret_cast<uint4v*>(&K_s[key * KLD + dc * 8]) = val;
     }
-    // V: 8 groups of 4 keys; a 16-byte word = 2 value columns x 4 keys, straight into two V^T rows
-    for (int c = tid; c < 8 * (DV / 2); c += 256) {
+    // V: 8 groups of 4 keys; a 16-byte word = 2 value columns x 4 keys
+#pragma unroll
+    for (int u = 0; u < VCH; ++u) {
+      const int c = tid + 256 * u;
       const int kg = c / (DV / 2), dc = c % (DV / 2);
       const int j = kt * 32 + 4 * kg;
-      uint4v val = uint4v{0u, 0u, 0u, 0u};
-      if (j <= j_hi) {
+      vreg[u] = uint4v{0u, 0u, 0u, 0u};
+      if (c < 8 * (DV / 2) && j <= j_hi) {
         const long long page = table[j / BS];
-        val = *reinterpret_cast<const uint4v*>(p.v_cache + page * p.vb_stride + (long long)((j % BS) >> 2) * (4LL * G * DV) +
-                                               4LL * (g * DV + 2 * dc));
+        vreg[u] = *reinterpret_cast<const uint4v*>(p.v_cache + page * p.vb_stride + (long long)((j % BS) >> 2) * (4LL * G * DV) +
+                                                   4LL * (g * DV + 2 * dc));
       }
-      typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
-      *reinterpret_cast<uint2v*>(&Vt_s[(2 * dc) * kVPad + 4 * kg]) = uint2v{val[0], val[1]};
-      *reinterpret_cast<uint2v*>(&Vt_s[(2 * dc + 1) * kVPad + 4 * kg]) = uint2v{val[2], val[3]};
     }
+    if (tid < 96) {
+      const int dist = pos0 - kt * 32 - 31 + tid;  // (row - key + 31) = tid
+      breg = dist >= 0 && dist < p.window ? bias_h[dist] : 0.f;
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int u = 0; u < KCH; ++u) {
+      const int c = tid + 256 * u;
+      if (c < 32 * (D / 8)) *reinterpret_cast<uint4v*>(&K_s[(c / (D / 8)) * KLD + (c % (D / 8)) * 8]) = kreg[u];
+    }
+#pragma unroll
+    for (int u = 0; u < VCH; ++u) {
+      const int c = tid + 256 * u;
+      if (c < 8 * (DV / 2)) {
+        const int kg = c / (DV / 2), dc = c % (DV / 2);
+        *reinterpret_cast<uint2v*>(&Vt_s[(2 * dc) * kVPad + 4 * kg]) = uint2v{vreg[u][0], vreg[u][1]};
+        *reinterpret_cast<uint2v*>(&Vt_s[(2 * dc + 1) * kVPad + 4 * kg]) = uint2v{vreg[u][2], vreg[u][3]};
+      }
+    }
+    if (tid < 96) bias_s[tid] = breg;
+  };
+
+  const int kt_lo = j_lo / 32, kt_hi = j_hi / 32;
+  fetch(kt_lo);
+  for (int kt = kt_lo; kt <= kt_hi; ++kt) {
     __syncthreads();
+    stash();
+    __syncthreads();
+    if (kt < kt_hi) fetch(kt + 1);
     // the tile's keys [32 kt, 32 kt + 31] against this wave's rows: nothing visible -> nothing to do
     if (!wave_live || kt * 32 > w_max || kt * 32 + 31 < w_min - p.window + 1) continue;
 
@@ -293,25 +327,35 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
         sacc[sub] = mfma16(a, qlo[kd], sacc[sub]);
       }
     }
+    // every key of the tile visible to every row of the wave: no masks
+    const bool inner = kt * 32 + 31 <= w_min && kt * 32 >= w_max - p.window + 1 && w_max - w_min == 15;
     float s[8];
-    bool ok[8];
     float mx = -1e30f;
+    if (inner) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int j = kt * 32 + (e >> 2) * 16 + 4 * g4 + (e & 3);
-      const int dist = i_q - j;
-      ok[e] = q_valid && dist >= 0 && dist < p.window;
-      s[e] = ok[e] ? sacc[e >> 2][e & 3] - bias_h[dist] : -1e30f;
-      mx = fmaxf(mx, s[e]);
+      for (int e = 0; e < 8; ++e) {
+        const int jl = (e >> 2) * 16 + 4 * g4 + (e & 3);
+        s[e] = sacc[e >> 2][e & 3] - bias_s[qrow - jl + 31];
+        mx = fmaxf(mx, s[e]);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int jl = (e >> 2) * 16 + 4 * g4 + (e & 3);
+        const int dist = i_q - (kt * 32 + jl);
+        const bool ok = q_valid && dist >= 0 && dist < p.window;
+        s[e] = ok ? sacc[e >> 2][e & 3] - bias_s[qrow - jl + 31] : -1e30f;
+        mx = fmaxf(mx, s[e]);
+      }
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m, mx);
-    const float alpha = expf(m - m_new);
+    const float alpha = __expf(m - m_new);
     float pe[8], psum = 0.f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      pe[e] = ok[e] ? expf(s[e] - m_new) : 0.f;
+      pe[e] = s[e] > -1e29f ? __expf(s[e] - m_new) : 0.f;
       psum += pe[e];
     }
     psum += __shfl_xor(psum, 16, 64);
@@ -328,10 +372,16 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
     float ar[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) ar[r] = __shfl(alpha, 4 * g4 + r, 64);
+    // (the running maxima settle after the first tiles: most tiles rescale nothing)
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int n = 0; n < NV; ++n) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) O[n][r] *= ar[r];
+      }
+    }
 #pragma unroll
     for (int n = 0; n < NV; ++n) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) O[n][r] *= ar[r];
       const bf16_t* vrow = &Vt_s[(n * 16 + r16) * kVPad];
       const short4v b0 = *reinterpret_cast<const short4v*>(vrow + 4 * g4);
       const short4v b1 = *reinterpret_cast<const short4v*>(vrow + 16 + 4 * g4);
@@ -389,216 +439,4 @@ extern "C" int r32_window_attn_mfma(const float* q, const void* k_cache, const v
     case 4: return launch_mfma_nv<4>(p, Dv / 16, grid, s);
   }
   return -1;
-}
-
-// ---------------------------------------------------------------------------------------------------------
-// window_attn_decode_kernel: one new token per sequence on the matrix cores (bf16 cache), split over the keys.
-//
-// One wave per (sequence b, key/value head g, head chunk, key split).  The N = 16 columns of the MFMA are the
-// (up to 16) query heads that share head g, so K and V are read ONCE for all of them, straight from the paged
-// cache into the operands — no LDS: a K row's 16 bytes are an A operand as they lie, the interleaved V word is a
-// B operand as it lies.  Same arithmetic as the portion kernel (hi + lo halves of q and of the weights, bias
-// table, fp32 online softmax).  Each split leaves an unnormalised partial (o, m, l); the reduce kernel merges
-// them (splits == 1: still through the reduce, which then only normalises).
-struct WAttnDecodeParams {
-  const float* q;          // [B, H*D]
-  const bf16_t* k_cache;
-  const bf16_t* v_cache;
-  long long kb_stride, vb_stride;
-  int block_size;
-  const int* positions;    // [B]: the new token's position (its key is already in the cache)
-  const int* block_tables;
-  int bt_width;
-  const float* bias;       // [H, window]
-  int window;
-  float* part_o;           // [B, H, S, Dv]
-  float* part_ml;          // [B, H, S, 2]
-  int H, G, S, keys_per_split;  // keys_per_split: a multiple of 32
-};
-
-template <int ND, int NV>
-__global__ void __launch_bounds__(64) window_attn_decode_kernel(const WAttnDecodeParams p) {
-  constexpr int D = 32 * ND, DV = 16 * NV;
-  const int b = blockIdx.x, split = blockIdx.z;
-  const int H = p.H, G = p.G, Hg = H / G, chunks = (Hg + 15) / 16;
-  const int g = blockIdx.y / chunks, h0 = g * Hg + (blockIdx.y % chunks) * 16;
-  const int nh = min(16, g * Hg + Hg - h0);  // heads of this chunk
-  const int lane = threadIdx.x, r16 = lane & 15, g4 = lane >> 4;
-  const int i = p.positions[b];
-  const int j_lo = max(0, i - p.window + 1);
-  const int base = (j_lo / 32) * 32 + split * p.keys_per_split;  // this split's first key (a multiple of 32)
-  const int last = min(i, base + p.keys_per_split - 1);
-  const int* table = p.block_tables + (size_t)b * p.bt_width;
-  const int BS = p.block_size;
-  const bool h_valid = r16 < nh;
-  const int h = h0 + (h_valid ? r16 : 0);
-
-  short8 qhi[ND], qlo[ND];
-#pragma unroll
-  for (int kd = 0; kd < ND; ++kd) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      float x = 0.f;
-      if (h_valid) x = p.q[((size_t)b * H + h) * D + kd * 32 + 8 * g4 + e];
-      const bf16_t hi = f2bf(x);
-      qhi[kd][e] = (short)hi;
-      qlo[kd][e] = (short)f2bf(x - bf2f(hi));
-    }
-  }
-  float4v O[NV];
-#pragma unroll
-  for (int n = 0; n < NV; ++n) O[n] = float4v{0.f, 0.f, 0.f, 0.f};
-  float m = -1e30f, l = 0.f;
-  const float* bias_h = p.bias + (size_t)h * p.window;
-
-  for (int t0 = base; t0 <= last; t0 += 32) {
-    float4v sacc[2];
-#pragma unroll
-    for (int sub = 0; sub < 2; ++sub) {
-      sacc[sub] = float4v{0.f, 0.f, 0.f, 0.f};
-      const int j = min(t0 + sub * 16 + r16, i);  // (rows past the token are masked below: any valid row does)
-      const bf16_t* kr = p.k_cache + (long long)table[j / BS] * p.kb_stride + ((long long)(j % BS) * G + g) * D + 8 * g4;
-#pragma unroll
-      for (int kd = 0; kd < ND; ++kd) {
-        const short8 a = *reinterpret_cast<const short8*>(kr + kd * 32);
-        sacc[sub] = mfma16(a, qhi[kd], sacc[sub]);
-        sacc[sub] = mfma16(a, qlo[kd], sacc[sub]);
-      }
-    }
-    float s[8];
-    bool ok[8];
-    float mx = -1e30f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int j = t0 + (e >> 2) * 16 + 4 * g4 + (e & 3);
-      const int dist = i - j;
-      ok[e] = h_valid && dist >= 0 && dist < p.window && j <= last;
-      s[e] = ok[e] ? sacc[e >> 2][e & 3] - bias_h[dist] : -1e30f;
-      mx = fmaxf(mx, s[e]);
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m, mx);
-    const float alpha = expf(m - m_new);
-    float pe[8], psum = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      pe[e] = ok[e] ? expf(s[e] - m_new) : 0.f;
-      psum += pe[e];
-    }
-    psum += __shfl_xor(psum, 16, 64);
-    psum += __shfl_xor(psum, 32, 64);
-    l = l * alpha + psum;
-    m = m_new;
-    short8 ph, pl;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const bf16_t hi = f2bf(pe[e]);
-      ph[e] = (short)hi;
-      pl[e] = (short)f2bf(pe[e] - bf2f(hi));
-    }
-    float ar[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) ar[r] = __shfl(alpha, 4 * g4 + r, 64);
-    // the lane's two 4-key groups: keys t0 + 4 g4 .. and t0 + 16 + 4 g4 .. (groups past the token: any valid one,
-    // their weights are 0)
-    const int ja = min(t0 + 4 * g4, (i / 4) * 4), jb = min(t0 + 16 + 4 * g4, (i / 4) * 4);
-    const bf16_t* va = p.v_cache + (long long)table[ja / BS] * p.vb_stride + (long long)((ja % BS) >> 2) * (4LL * G * DV) + 4LL * (g * DV + r16);
-    const bf16_t* vb = p.v_cache + (long long)table[jb / BS] * p.vb_stride + (long long)((jb % BS) >> 2) * (4LL * G * DV) + 4LL * (g * DV + r16);
-#pragma unroll
-    for (int n = 0; n < NV; ++n) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) O[n][r] *= ar[r];
-      const short4v b0 = *reinterpret_cast<const short4v*>(va + 64 * n);
-      const short4v b1 = *reinterpret_cast<const short4v*>(vb + 64 * n);
-      const short8 bb = short8{b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
-      O[n] = mfma16(ph, bb, O[n]);
-      O[n] = mfma16(pl, bb, O[n]);
-    }
-  }
-  // partials: O rows are heads 4 g4 + r, columns dv 16 n + r16
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int hr = 4 * g4 + r;
-    if (hr < nh) {
-      float* po = p.part_o + (((size_t)b * H + h0 + hr) * p.S + split) * DV;
-#pragma unroll
-      for (int n = 0; n < NV; ++n) po[n * 16 + r16] = O[n][r];
-    }
-  }
-  if (g4 == 0 && h_valid) {
-    float* pm = p.part_ml + (((size_t)b * H + h) * p.S + split) * 2;
-    pm[0] = m;
-    pm[1] = l;
-  }
-}
-
-// out[b, h, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s  (splits that saw no key have l = 0)
-__global__ void window_attn_reduce_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                          bf16_t* __restrict__ out, int ldo, int H, int S, int Dv) {
-  const int b = blockIdx.x, h = blockIdx.y;
-  const float* ml = part_ml + ((size_t)b * H + h) * S * 2;
-  float M = -1e30f;
-  for (int s = 0; s < S; ++s)
-    if (ml[2 * s + 1] > 0.f) M = fmaxf(M, ml[2 * s]);
-  float L = 0.f;
-  for (int s = 0; s < S; ++s)
-    if (ml[2 * s + 1] > 0.f) L += expf(ml[2 * s] - M) * ml[2 * s + 1];
-  const float inv = L > 0.f ? 1.0f / L : 0.f;
-  for (int dv = threadIdx.x; dv < Dv; dv += blockDim.x) {
-    float acc = 0.f;
-    for (int s = 0; s < S; ++s)
-      if (ml[2 * s + 1] > 0.f) acc += expf(ml[2 * s] - M) * part_o[(((size_t)b * H + h) * S + s) * Dv + dv];
-    out[(size_t)b * ldo + (size_t)h * Dv + dv] = f2bf(acc * inv);
-  }
-}
-
-template <int ND>
-int launch_decode_nv(const WAttnDecodeParams& p, int nv, dim3 grid, hipStream_t s) {
-  switch (nv) {
-    case 2: window_attn_decode_kernel<ND, 2><<<grid, 64, 0, s>>>(p); break;
-    case 4: window_attn_decode_kernel<ND, 4><<<grid, 64, 0, s>>>(p); break;
-    case 8: window_attn_decode_kernel<ND, 8><<<grid, 64, 0, s>>>(p); break;
-    default: return -1;
-  }
-  return (int)hipGetLastError();
-}
-
-// Splits for a decode step of B sequences whose windows hold at most max_keys keys: enough waves to fill the chip,
-// at least 64 keys each.
-extern "C" int r32_window_attn_decode_splits(int B, int G, int Hg, int max_keys) {
-  const int waves = B * G * ((Hg + 15) / 16);
-  int s = (2048 + waves - 1) / waves;
-  const int by_keys = (max_keys + 32 + 63) / 64;
-  if (s > by_keys) s = by_keys;
-  if (s > 64) s = 64;
-  return s < 1 ? 1 : s;
-}
-
-// part_o: fp32 [B * H * S * Dv], part_ml: fp32 [B * H * S * 2] scratch of the caller.  max_keys: an upper bound of
-// the keys any row sees (min(window, longest context)), known on the host.
-extern "C" int r32_window_attn_decode(const float* q, const void* k_cache, const void* v_cache, long long kb_stride,
-                                      long long vb_stride, int block_size, const int* positions, const int* block_tables,
-                                      int bt_width, const float* bias, int window, float* part_o, float* part_ml, int S,
-                                      int max_keys, void* out, int ldo, int B, int H, int G, int D, int Dv, hipStream_t s) {
-  if (B <= 0) return 0;
-  if (!r32_window_attn_mfma_ok(D, Dv) || H % G != 0 || S < 1) return -1;
-  WAttnDecodeParams p;
-  p.q = q; p.k_cache = (const bf16_t*)k_cache; p.v_cache = (const bf16_t*)v_cache; p.kb_stride = kb_stride;
-  p.vb_stride = vb_stride; p.block_size = block_size; p.positions = positions; p.block_tables = block_tables;
-  p.bt_width = bt_width; p.bias = bias; p.window = window; p.part_o = part_o; p.part_ml = part_ml; p.H = H; p.G = G;
-  p.S = S;
-  // a row's keys start at a multiple of 32 at or below its window's first key: up to max_keys + 31 keys to cover
-  p.keys_per_split = (((max_keys + 31 + S - 1) / S) + 31) / 32 * 32;
-  const int Hg = H / G;
-  const dim3 grid(B, G * ((Hg + 15) / 16), S);
-  int rc = -1;
-  switch (D / 32) {
-    case 1: rc = launch_decode_nv<1>(p, Dv / 16, grid, s); break;
-    case 2: rc = launch_decode_nv<2>(p, Dv / 16, grid, s); break;
-    case 4: rc = launch_decode_nv<4>(p, Dv / 16, grid, s); break;
-  }
-  if (rc != 0) return rc;
-  window_attn_reduce_kernel<<<dim3(B, H), 64, 0, s>>>(part_o, part_ml, (bf16_t*)out, ldo, H, S, Dv);
-  return (int)hipGetLastError();
 }

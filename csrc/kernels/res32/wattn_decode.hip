@@ -1,0 +1,224 @@
+// Decode rows of the sliding-window attention (see wattn.hip for the scores, the cache layout and the portion kernel).
+#include "../common.h"
+
+using namespace lwc;
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+
+LWC_DEVICE float4v mfma16(const short8& a, const short8& b, const float4v& c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+extern "C" int r32_window_attn_mfma_ok(int D, int Dv);
+
+// ---------------------------------------------------------------------------------------------------------
+// window_attn_decode_kernel: one new token per sequence on the matrix cores (bf16 cache), split over the keys.
+//
+// One wave per (sequence b, key/value head g, head chunk, key split).  The N = 16 columns of the MFMA are the
+// (up to 16) query heads that share head g, so K and V are read ONCE for all of them, straight from the paged
+// cache into the operands — no LDS: a K row's 16 bytes are an A operand as they lie, the interleaved V word is a
+// B operand as it lies.  Same arithmetic as the portion kernel (hi + lo halves of q and of the weights, bias
+// table, fp32 online softmax).  Each split leaves an unnormalised partial (o, m, l); the reduce kernel merges
+// them (splits == 1: still through the reduce, which then only normalises).
+struct WAttnDecodeParams {
+  const float* q;          // [B, H*D]
+  const bf16_t* k_cache;
+  const bf16_t* v_cache;
+  long long kb_stride, vb_stride;
+  int block_size;
+  const int* positions;    // [B]: the new token's position (its key is already in the cache)
+  const int* block_tables;
+  int bt_width;
+  const float* bias;       // [H, window]
+  int window;
+  float* part_o;           // [B, H, S, Dv]
+  float* part_ml;          // [B, H, S, 2]
+  int H, G, S, keys_per_split;  // keys_per_split: a multiple of 32
+};
+
+template <int ND, int NV>
+__global__ void __launch_bounds__(64) window_attn_decode_kernel(const WAttnDecodeParams p) {
+  constexpr int D = 32 * ND, DV = 16 * NV;
+  const int b = blockIdx.x, split = blockIdx.z;
+  const int H = p.H, G = p.G, Hg = H / G, chunks = (Hg + 15) / 16;
+  const int g = blockIdx.y / chunks, h0 = g * Hg + (blockIdx.y % chunks) * 16;
+  const int nh = min(16, g * Hg + Hg - h0);  // heads of this chunk
+  const int lane = threadIdx.x, r16 = lane & 15, g4 = lane >> 4;
+  const int i = p.positions[b];
+  const int j_lo = max(0, i - p.window + 1);
+  const int base = (j_lo / 32) * 32 + split * p.keys_per_split;  // this split's first key (a multiple of 32)
+  const int last = min(i, base + p.keys_per_split - 1);
+  const int* table = p.block_tables + (size_t)b * p.bt_width;
+  const int BS = p.block_size;
+  const bool h_valid = r16 < nh;
+  const int h = h0 + (h_valid ? r16 : 0);
+
+  short8 qhi[ND], qlo[ND];
+#pragma unroll
+  for (int kd = 0; kd < ND; ++kd) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float x = 0.f;
+      if (h_valid) x = p.q[((size_t)b * H + h) * D + kd * 32 + 8 * g4 + e];
+      const bf16_t hi = f2bf(x);
+      qhi[kd][e] = (short)hi;
+      qlo[kd][e] = (short)f2bf(x - bf2f(hi));
+    }
+  }
+  float4v O[NV];
+#pragma unroll
+  for (int n = 0; n < NV; ++n) O[n] = float4v{0.f, 0.f, 0.f, 0.f};
+  float m = -1e30f, l = 0.f;
+  const float* bias_h = p.bias + (size_t)h * p.window;
+
+  for (int t0 = base; t0 <= last; t0 += 32) {
+    float4v sacc[2];
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      sacc[sub] = float4v{0.f, 0.f, 0.f, 0.f};
+      const int j = min(t0 + sub * 16 + r16, i);  // (rows past the token are masked below: any valid row does)
+      const bf16_t* kr = p.k_cache + (long long)table[j / BS] * p.kb_stride + ((long long)(j % BS) * G + g) * D + 8 * g4;
+#pragma unroll
+      for (int kd = 0; kd < ND; ++kd) {
+        const short8 a = *reinterpret_cast<const short8*>(kr + kd * 32);
+        sacc[sub] = mfma16(a, qhi[kd], sacc[sub]);
+        sacc[sub] = mfma16(a, qlo[kd], sacc[sub]);
+      }
+    }
+    float s[8];
+    bool ok[8];
+    float mx = -1e30f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int j = t0 + (e >> 2) * 16 + 4 * g4 + (e & 3);
+      const int dist = i - j;
+      ok[e] = h_valid && dist >= 0 && dist < p.window && j <= last;
+      s[e] = ok[e] ? sacc[e >> 2][e & 3] - bias_h[dist] : -1e30f;
+      mx = fmaxf(mx, s[e]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float alpha = expf(m - m_new);
+    float pe[8], psum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      pe[e] = ok[e] ? expf(s[e] - m_new) : 0.f;
+      psum += pe[e];
+    }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * alpha + psum;
+    m = m_new;
+    short8 ph, pl;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const bf16_t hi = f2bf(pe[e]);
+      ph[e] = (short)hi;
+      pl[e] = (short)f2bf(pe[e] - bf2f(hi));
+    }
+    float ar[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) ar[r] = __shfl(alpha, 4 * g4 + r, 64);
+    // the lane's two 4-key groups: keys t0 + 4 g4 .. and t0 + 16 + 4 g4 .. (groups past the token: any valid one,
+    // their weights are 0)
+    const int ja = min(t0 + 4 * g4, (i / 4) * 4), jb = min(t0 + 16 + 4 * g4, (i / 4) * 4);
+    const bf16_t* va = p.v_cache + (long long)table[ja / BS] * p.vb_stride + (long long)((ja % BS) >> 2) * (4LL * G * DV) + 4LL * (g * DV + r16);
+    const bf16_t* vb = p.v_cache + (long long)table[jb / BS] * p.vb_stride + (long long)((jb % BS) >> 2) * (4LL * G * DV) + 4LL * (g * DV + r16);
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) O[n][r] *= ar[r];
+      const short4v b0 = *reinterpret_cast<const short4v*>(va + 64 * n);
+      const short4v b1 = *reinterpret_cast<const short4v*>(vb + 64 * n);
+      const short8 bb = short8{b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+      O[n] = mfma16(ph, bb, O[n]);
+      O[n] = mfma16(pl, bb, O[n]);
+    }
+  }
+  // partials: O rows are heads 4 g4 + r, columns dv 16 n + r16
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int hr = 4 * g4 + r;
+    if (hr < nh) {
+      float* po = p.part_o + (((size_t)b * H + h0 + hr) * p.S + split) * DV;
+#pragma unroll
+      for (int n = 0; n < NV; ++n) po[n * 16 + r16] = O[n][r];
+    }
+  }
+  if (g4 == 0 && h_valid) {
+    float* pm = p.part_ml + (((size_t)b * H + h) * p.S + split) * 2;
+    pm[0] = m;
+    pm[1] = l;
+  }
+}
+
+// out[b, h, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s  (splits that saw no key have l = 0)
+__global__ void window_attn_reduce_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                          bf16_t* __restrict__ out, int ldo, int H, int S, int Dv) {
+  const int b = blockIdx.x, h = blockIdx.y;
+  const float* ml = part_ml + ((size_t)b * H + h) * S * 2;
+  float M = -1e30f;
+  for (int s = 0; s < S; ++s)
+    if (ml[2 * s + 1] > 0.f) M = fmaxf(M, ml[2 * s]);
+  float L = 0.f;
+  for (int s = 0; s < S; ++s)
+    if (ml[2 * s + 1] > 0.f) L += expf(ml[2 * s] - M) * ml[2 * s + 1];
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
+  for (int dv = threadIdx.x; dv < Dv; dv += blockDim.x) {
+    float acc = 0.f;
+    for (int s = 0; s < S; ++s)
+      if (ml[2 * s + 1] > 0.f) acc += expf(ml[2 * s] - M) * part_o[(((size_t)b * H + h) * S + s) * Dv + dv];
+    out[(size_t)b * ldo + (size_t)h * Dv + dv] = f2bf(acc * inv);
+  }
+}
+
+template <int ND>
+int launch_decode_nv(const WAttnDecodeParams& p, int nv, dim3 grid, hipStream_t s) {
+  switch (nv) {
+    case 2: window_attn_decode_kernel<ND, 2><<<grid, 64, 0, s>>>(p); break;
+    case 4: window_attn_decode_kernel<ND, 4><<<grid, 64, 0, s>>>(p); break;
+    case 8: window_attn_decode_kernel<ND, 8><<<grid, 64, 0, s>>>(p); break;
+    default: return -1;
+  }
+  return (int)hipGetLastError();
+}
+
+// Splits for a decode step of B sequences whose windows hold at most max_keys keys: enough waves to fill the chip,
+// at least 64 keys each.
+extern "C" int r32_window_attn_decode_splits(int B, int G, int Hg, int max_keys) {
+  const int waves = B * G * ((Hg + 15) / 16);
+  int s = (2048 + waves - 1) / waves;
+  const int by_keys = (max_keys + 32 + 63) / 64;
+  if (s > by_keys) s = by_keys;
+  if (s > 64) s = 64;
+  return s < 1 ? 1 : s;
+}
+
+// part_o: fp32 [B * H * S * Dv], part_ml: fp32 [B * H * S * 2] scratch of the caller.  max_keys: an upper bound of
+// the keys any row sees (min(window, longest context)), known on the host.
+extern "C" int r32_window_attn_decode(const float* q, const void* k_cache, const void* v_cache, long long kb_stride,
+                                      long long vb_stride, int block_size, const int* positions, const int* block_tables,
+                                      int bt_width, const float* bias, int window, float* part_o, float* part_ml, int S,
+                                      int max_keys, void* out, int ldo, int B, int H, int G, int D, int Dv, hipStream_t s) {
+  if (B <= 0) return 0;
+  if (!r32_window_attn_mfma_ok(D, Dv) || H % G != 0 || S < 1) return -1;
+  WAttnDecodeParams p;
+  p.q = q; p.k_cache = (const bf16_t*)k_cache; p.v_cache = (const bf16_t*)v_cache; p.kb_stride = kb_stride;
+  p.vb_stride = vb_stride; p.block_size = block_size; p.positions = positions; p.block_tables = block_tables;
+  p.bt_width = bt_width; p.bias = bias; p.window = window; p.part_o = part_o; p.part_ml = part_ml; p.H = H; p.G = G;
+  p.S = S;
+  // a row's keys start at a multiple of 32 at or below its window's first key: up to max_keys + 31 keys to cover
+  p.keys_per_split = (((max_keys + 31 + S - 1) / S) + 31) / 32 * 32;
+  const int Hg = H / G;
+  const dim3 grid(B, G * ((Hg + 15) / 16), S);
+  int rc = -1;
+  switch (D / 32) {
+    case 1: rc = launch_decode_nv<1>(p, Dv / 16, grid, s); break;
+    case 2: rc = launch_decode_nv<2>(p, Dv / 16, grid, s); break;
+    case 4: rc = launch_decode_nv<4>(p, Dv / 16, grid, s); break;
+  }
+  if (rc != 0) return rc;
+  window_attn_reduce_kernel<<<dim3(B, H), 64, 0, s>>>(part_o, part_ml, (bf16_t*)out, ldo, H, S, Dv);
+  return (int)hipGetLastError();
+}

@@ -67,7 +67,8 @@ def _torch_flags(name: str = "_kernels") -> tuple[list[str], list[str]]:
 # Per-kernel-file code generation flags.  The attention kernels keep their accumulators in VGPRs (the
 # compiler's default AGPR form moved every O accumulator AGPR <-> VGPR around each MFMA: 72 v_accvgpr per
 # 32-key tile).
-PER_FILE_FLAGS = {f: ["-mllvm", "-amdgpu-mfma-vgpr-form=1"] for f in ("attention_prefill.hip", "attention_decode.hip")}
+PER_FILE_FLAGS = {f: ["-mllvm", "-amdgpu-mfma-vgpr-form=1"] for f in ("attention_prefill.hip", "attention_decode.hip",
+                                                                      "wattn.hip")}
 
 
 def build_kernels(jobs: int = 8, force: bool = False) -> Path:
@@ -120,7 +121,7 @@ def build_res32(jobs: int = 8, force: bool = False) -> Path:
         obj = obj_dir / (src.stem + ".o")
         objs.append(obj)
         if force or _stale(obj, [src, *headers]):
-            jobs_list.append(base + ["-c", str(src), "-o", str(obj)])
+            jobs_list.append(base + PER_FILE_FLAGS.get(src.name, []) + ["-c", str(src), "-o", str(obj)])
     bsrc, bobj = kdir / "bindings.cpp", obj_dir / "bindings.o"
     objs.append(bobj)
     if force or _stale(bobj, [bsrc]):

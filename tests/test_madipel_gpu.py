@@ -67,6 +67,12 @@ def test_xielu_and_residual(gpu, dtype, tol):
     got = out.cpu().double()
     assert ((got[:, 20:84] - ref).abs() / (1 + ref.abs())).max() < tol
     assert got[:, :20].abs().max() == 0 and got[:, 84:].abs().max() == 0
+    # rows whose width and leading dimensions are multiples of 8 (the 16-byte path in bf16)
+    wide2, out2 = torch.zeros(5, 128, dtype=dtype, device=gpu), torch.zeros(5, 96, dtype=dtype, device=gpu)
+    wide2[:, 16:80] = _dev(z, dtype)
+    res32.xielu(wide2[:, 16:80], _dev(pq, dtype), out2[:, 32:96])
+    assert ((out2.cpu().double()[:, 32:96] - ref).abs() / (1 + ref.abs())).max() < tol
+    assert out2[:, :32].abs().max() == 0
     x = torch.randn(5, 64, generator=g)
     xd = x.to(gpu)
     res32.residual_add_scaled(xd, _dev(z, dtype), 0.37)
