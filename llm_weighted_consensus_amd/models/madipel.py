@@ -20,7 +20,9 @@ Value blending: the first layer whose config says ``v_mix`` publishes its values
 rows); every later such layer caches ``(1 - lam) v + lam v0``.  v0 lives only inside one forward.
 
 ``dtype=torch.float32`` runs every GEMM, activation and the cache in true fp32 (exact mode); bf16 is the serving
-mode.  GEMMs are the vendor library's (torch -> hipBLASLt), as for the other decoders' untuned shapes.
+mode.  GEMMs go through the per-shape planner of the other decoders (``ops/gemm_plan.py``): the vendor library
+(torch -> hipBLASLt) for untuned shapes and for fp32, and for a decode bucket whichever of the library and the
+hand-written cores was timed faster before the bucket's hipGraph is captured (:meth:`MadipelModel.tune_gemms`).
 """
 from __future__ import annotations
 
@@ -32,7 +34,8 @@ from typing import Callable, List, Optional
 import torch
 import torch.nn.functional as F
 
-from ..ops import res32
+from .. import ops
+from ..ops import gemm_plan, res32
 from .cache import PagedLayerCache
 from .config import MadipelConfig
 
@@ -77,6 +80,7 @@ class MadipelModel:
         self.inv_freq = res32.sinpos_inv_freq(cfg.hidden, cfg.sinpos_base, self.device)
         raw = self._read(weights_path) if weights_path else self._random(seed)
         self._assemble(raw)
+        self.g8_ws = None  # the hand-written GEMM cores' workspace, made when a shape is first tuned
         # called with (layer index, residual stream) after every layer when set (bring-up, tests)
         self.on_layer: Optional[Callable[[int, torch.Tensor], None]] = None
 
@@ -172,6 +176,31 @@ class MadipelModel:
             if dt == torch.bfloat16 and m.heads * m.window <= (1 << 26) and res32.kernels().window_attn_mfma_ok(m.dim, m.vdim):
                 Lw.bias = res32.distance_bias(Lw.r1, Lw.r2, m.window)
 
+    # ------------------------------------------------------------------ GEMMs
+    def _linear(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+        if self.g8_ws is not None:
+            return gemm_plan.linear(x, w, ws=self.g8_ws)
+        return F.linear(x, w)
+
+    def tune_gemms(self, M: int, bucket: bool = False, lm_head: bool = True, only=None) -> None:
+        """Pick the backend of every projection at M rows by timing the library and the hand-written cores (the
+        engine calls this before it captures a decode bucket's graph).  bf16 only, and only where the full kernel
+        extension is built; otherwise every GEMM stays on the library."""
+        if self.dtype != torch.bfloat16 or only is not None or not ops.available():
+            return
+        if self.g8_ws is None:
+            self.g8_ws = ops.new_gemm8p_workspace(self.device)
+        seen = set()
+        for L in self.layers:
+            for w in (L.w_in, L.w_out):
+                if tuple(w.shape) not in seen:
+                    seen.add(tuple(w.shape))
+                    x = torch.randn(M, w.shape[1], device=self.device).to(self.dtype)
+                    gemm_plan.tune(x, w, ws=self.g8_ws, bucket=bucket)
+        if lm_head:
+            gemm_plan.tune(torch.randn(M, self.cfg.hidden, device=self.device).to(self.dtype), self.head, ws=self.g8_ws,
+                           bucket=bucket)
+
     # ------------------------------------------------------------------ cache
     def _layer_dims(self):
         return [(L.mixer.nk, L.mixer.nv) for L in self.cfg.layer_specs]
@@ -193,7 +222,7 @@ class MadipelModel:
         for li, (S, L) in enumerate(zip(cfg.layer_specs, self.layers)):
             m = S.mixer
             h = res32.layernorm(x, L.norm_w, L.norm_b, cfg.norm_eps)
-            proj = F.linear(h, L.w_in)
+            proj = self._linear(h, L.w_in)
             if L.vmode and v0 is None:
                 v0 = torch.empty(T, m.nv, dtype=torch.float32, device=x.device)
             q = res32.proj_norm_kv_write(proj, L.q_norm, L.k_norm, L.head_scale, slots, cache.k[li], cache.v[li],
@@ -203,14 +232,14 @@ class MadipelModel:
             attend(q, li, cat[:, :no])
             if S.mlp_kind:
                 res32.xielu(proj[:, m.nq + m.nk + m.nv:], L.act, cat[:, no:])
-            res32.residual_add_scaled(x, F.linear(cat, L.w_out), cfg.residual_mult)
+            res32.residual_add_scaled(x, self._linear(cat, L.w_out), cfg.residual_mult)
             if self.on_layer is not None:
                 self.on_layer(li, x)
         return x
 
     def _logits(self, x: torch.Tensor, rows: Optional[torch.Tensor], float_logits: bool) -> torch.Tensor:
         h = res32.layernorm(x, self.final_w, self.final_b, self.cfg.norm_eps, rows=rows)
-        lg = F.linear(h, self.head).float() * self.cfg.logit_scale
+        lg = self._linear(h, self.head).float() * self.cfg.logit_scale
         if float_logits:
             return lg
         V, Vp = self.cfg.vocab_size, self.logit_width
