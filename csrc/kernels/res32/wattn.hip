@@ -217,6 +217,7 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
   __shared__ __attribute__((aligned(16))) bf16_t K_s[32 * KLD];
   __shared__ __attribute__((aligned(16))) bf16_t Vt_s[DV * kVPad];
   __shared__ float bias_s[96];  // the tile's bias by (row - key + 31): rows 0..63 of the workgroup, keys 0..31 of the tile
+  extern __shared__ int pages_s[];  // the item's block table over this workgroup's key range (dynamic size)
   const int it = blockIdx.x / p.tiles_per_item, tile = blockIdx.x % p.tiles_per_item;
   const int q_begin = p.cu_q[it], q_end = p.cu_q[it + 1];
   const int row0 = q_begin + tile * 64;
@@ -255,6 +256,7 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
   float m = -1e30f, l = 0.f;
   const float* bias_h = p.bias + (size_t)h * p.window;
 
+  const int pg0 = ((j_lo / 32) * 32) / BS;  // first page of the workgroup's key range
   // a tile's words are fetched into registers one tile ahead (the loads fly while the previous tile is computed)
   uint4v kreg[KCH], vreg[VCH];
   float breg = 0.f;
@@ -266,7 +268,7 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
       const int j = kt * 32 + key;
       kreg[u] = uint4v{0u, 0u, 0u, 0u};
       if (c < 32 * (D / 8) && j <= j_hi) {
-        const long long page = table[j / BS];
+        const long long page = pages_s[j / BS - pg0];
         kreg[u] = *reinterpret_cast<const uint4v*>(p.k_cache + page * p.kb_stride + ((long long)(j % BS) * G + g) * D + dc * 8);
       }
     }
@@ -278,7 +280,7 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
       const int j = kt * 32 + 4 * kg;
       vreg[u] = uint4v{0u, 0u, 0u, 0u};
       if (c < 8 * (DV / 2) && j <= j_hi) {
-        const long long page = table[j / BS];
+        const long long page = pages_s[j / BS - pg0];
         vreg[u] = *reinterpret_cast<const uint4v*>(p.v_cache + page * p.vb_stride + (long long)((j % BS) >> 2) * (4LL * G * DV) +
                                                    4LL * (g * DV + 2 * dc));
       }
@@ -307,6 +309,10 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
   };
 
   const int kt_lo = j_lo / 32, kt_hi = j_hi / 32;
+  // the pages of keys [32 kt_lo, j_hi] once, so a tile's loads do not wait for a table lookup first
+  const int npg = j_hi / BS - pg0 + 1;
+  for (int c = tid; c < npg; c += 256) pages_s[c] = table[pg0 + c];
+  __syncthreads();
   fetch(kt_lo);
   for (int kt = kt_lo; kt <= kt_hi; ++kt) {
     __syncthreads();
@@ -405,11 +411,11 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
 }
 
 template <int ND>
-int launch_mfma_nv(const WAttnMfmaParams& p, int nv, dim3 grid, hipStream_t s) {
+int launch_mfma_nv(const WAttnMfmaParams& p, int nv, dim3 grid, size_t shm, hipStream_t s) {
   switch (nv) {
-    case 2: window_attn_mfma_kernel<ND, 2><<<grid, 256, 0, s>>>(p); break;
-    case 4: window_attn_mfma_kernel<ND, 4><<<grid, 256, 0, s>>>(p); break;
-    case 8: window_attn_mfma_kernel<ND, 8><<<grid, 256, 0, s>>>(p); break;
+    case 2: window_attn_mfma_kernel<ND, 2><<<grid, 256, shm, s>>>(p); break;
+    case 4: window_attn_mfma_kernel<ND, 4><<<grid, 256, shm, s>>>(p); break;
+    case 8: window_attn_mfma_kernel<ND, 8><<<grid, 256, shm, s>>>(p); break;
     default: return -1;
   }
   return (int)hipGetLastError();
@@ -433,10 +439,15 @@ extern "C" int r32_window_attn_mfma(const float* q, const void* k_cache, const v
   p.cu_q = cu_q; p.k_lens = k_lens; p.tiles_per_item = (max_q + 63) / 64; p.block_tables = block_tables;
   p.bt_width = bt_width; p.bias = bias; p.window = window; p.out = (bf16_t*)out; p.ldo = ldo; p.H = H; p.G = G;
   const dim3 grid(n_items * p.tiles_per_item, H);
+  // a workgroup's keys span at most window + 63 positions (from a 32-aligned start: + 31) and never more than the table
+  long long span = (long long)window + 63 + 31;
+  if (span > (long long)bt_width * block_size) span = (long long)bt_width * block_size;
+  const size_t shm = (size_t)(span / block_size + 2) * sizeof(int);
+  if (shm > 48 * 1024) return -2;
   switch (D / 32) {
-    case 1: return launch_mfma_nv<1>(p, Dv / 16, grid, s);
-    case 2: return launch_mfma_nv<2>(p, Dv / 16, grid, s);
-    case 4: return launch_mfma_nv<4>(p, Dv / 16, grid, s);
+    case 1: return launch_mfma_nv<1>(p, Dv / 16, grid, shm, s);
+    case 2: return launch_mfma_nv<2>(p, Dv / 16, grid, shm, s);
+    case 4: return launch_mfma_nv<4>(p, Dv / 16, grid, shm, s);
   }
   return -1;
 }
