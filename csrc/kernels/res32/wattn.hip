@@ -214,11 +214,13 @@ template <int ND, int NV>
 __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaParams p) {
   constexpr int D = 32 * ND, DV = 16 * NV, KLD = D + 8;
   constexpr int KCH = (32 * (D / 8) + 255) / 256, VCH = (8 * (DV / 2) + 255) / 256;  // 16-byte words per thread and tile
-  __shared__ __attribute__((aligned(16))) bf16_t K_s[32 * KLD];
-  __shared__ __attribute__((aligned(16))) bf16_t Vt_s[DV * kVPad];
-  __shared__ float bias_s[96];  // the tile's bias by (row - key + 31): rows 0..63 of the workgroup, keys 0..31 of the tile
+  // two images of every staged tile: tile kt + 1 is written while tile kt is read (one barrier per tile)
+  __shared__ __attribute__((aligned(16))) bf16_t K_s2[2][32 * KLD];
+  __shared__ __attribute__((aligned(16))) bf16_t Vt_s2[2][DV * kVPad];
+  __shared__ float bias_s2[2][96];  // the tile's bias by (row - key + 31): rows 0..63 of the workgroup, keys 0..31 of the tile
   extern __shared__ int pages_s[];  // the item's block table over this workgroup's key range (dynamic size)
-  const int it = blockIdx.x / p.tiles_per_item, tile = blockIdx.x % p.tiles_per_item;
+  // the last row tiles of an item see the most keys: they start first
+  const int it = blockIdx.x / p.tiles_per_item, tile = p.tiles_per_item - 1 - blockIdx.x % p.tiles_per_item;
   const int q_begin = p.cu_q[it], q_end = p.cu_q[it + 1];
   const int row0 = q_begin + tile * 64;
   if (row0 >= q_end) return;
@@ -290,7 +292,10 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
       breg = dist >= 0 && dist < p.window ? bias_h[dist] : 0.f;
     }
   };
-  auto stash = [&]() {
+  auto stash = [&](int buf) {
+    bf16_t* K_s = K_s2[buf];
+    bf16_t* Vt_s = Vt_s2[buf];
+    float* bias_s = bias_s2[buf];
 #pragma unroll
     for (int u = 0; u < KCH; ++u) {
       const int c = tid + 256 * u;
@@ -314,14 +319,16 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
   for (int c = tid; c < npg; c += 256) pages_s[c] = table[pg0 + c];
   __syncthreads();
   fetch(kt_lo);
+  stash(0);
+  __syncthreads();
   for (int kt = kt_lo; kt <= kt_hi; ++kt) {
-    __syncthreads();
-    stash();
-    __syncthreads();
+    const int cur = (kt - kt_lo) & 1;
+    const bf16_t* K_s = K_s2[cur];
+    const bf16_t* Vt_s = Vt_s2[cur];
+    const float* bias_s = bias_s2[cur];
     if (kt < kt_hi) fetch(kt + 1);
-    // the tile's keys [32 kt, 32 kt + 31] against this wave's rows: nothing visible -> nothing to do
-    if (!wave_live || kt * 32 > w_max || kt * 32 + 31 < w_min - p.window + 1) continue;
-
+    // the tile's keys [32 kt, 32 kt + 31] against this wave's rows: nothing visible -> nothing to compute
+    if (wave_live && kt * 32 <= w_max && kt * 32 + 31 >= w_min - p.window + 1) {
     float4v sacc[2];
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
@@ -395,6 +402,9 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
       O[n] = mfma16(ph, b, O[n]);
       O[n] = mfma16(pl, b, O[n]);
     }
+    }  // (this wave's work on the tile)
+    if (kt < kt_hi) stash(cur ^ 1);  // every wave left that image at the previous barrier
+    __syncthreads();
   }
   if (!wave_live) return;
 #pragma unroll
