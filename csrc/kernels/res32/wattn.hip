@@ -172,8 +172,8 @@ extern "C" int r32_window_attn(const float* q, const void* k_cache, const void* 
 // window_attn_mfma_kernel: prompt portions on the matrix cores (bf16 cache, D = 32 ND, Dv = 16 NV).
 //
 // Workgroup = 4 waves = 64 consecutive query rows of one (item, head); wave w owns rows 16w .. 16w+15 and all
-// four walk the 32-key tiles of the rows' windows, staged through LDS (K row-major, V transposed so that a
-// lane's four consecutive keys of one value column are one 8-byte read).  mfma_f32_16x16x32_bf16, lane l:
+// four walk the 32-key tiles of the rows' windows, staged through LDS (K row-major; V transposed with the keys
+// permuted so that a lane's eight k-slots of one value column are one 16-byte read).  mfma_f32_16x16x32_bf16, lane l:
 // r16 = l & 15, g = l >> 4:
 //   S^T = K Q^T : A = K rows from LDS, B = Q^T in registers; C reg r = S^T[key 4g + r][query r16], two 16-key
 //                 subtiles.  q is fp32: it enters as hi + lo bf16 halves (two MFMAs), so the scores keep fp32's
@@ -195,7 +195,7 @@ struct WAttnMfmaParams {
   const bf16_t* k_cache;
   const bf16_t* v_cache;
   long long kb_stride, vb_stride;
-  int block_size;
+  int block_size, bs_shift;  // block_size = 1 << bs_shift (the matrix-core kernels take power-of-two pages)
   const int* positions;
   const int* cu_q;
   const int* k_lens;
@@ -231,7 +231,10 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
   const int j_lo = max(0, pos0 - p.window + 1), j_hi = min(pos_last, k_len - 1);
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, r16 = lane & 15, g4 = lane >> 4;
   const int* table = p.block_tables + (size_t)it * p.bt_width;
-  const int BS = p.block_size;
+  const int BS = p.block_size, bsh = p.bs_shift;
+  // page and offset of key j (a runtime division would cost tens of instructions per load)
+  auto page_ix = [&](int j) { return j >> bsh; };
+  auto page_off = [&](int j) { return j & (BS - 1); };
   typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
 
   const int qrow = 16 * w + r16;
@@ -258,7 +261,7 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
   float m = -1e30f, l = 0.f;
   const float* bias_h = p.bias + (size_t)h * p.window;
 
-  const int pg0 = ((j_lo / 32) * 32) / BS;  // first page of the workgroup's key range
+  const int pg0 = page_ix((j_lo / 32) * 32);  // first page of the workgroup's key range
   // a tile's words are fetched into registers one tile ahead (the loads fly while the previous tile is computed)
   uint4v kreg[KCH], vreg[VCH];
   float breg = 0.f;
@@ -270,8 +273,8 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
       const int j = kt * 32 + key;
       kreg[u] = uint4v{0u, 0u, 0u, 0u};
       if (c < 32 * (D / 8) && j <= j_hi) {
-        const long long page = pages_s[j / BS - pg0];
-        kreg[u] = *reinterpret_cast<const uint4v*>(p.k_cache + page * p.kb_stride + ((long long)(j % BS) * G + g) * D + dc * 8);
+        const long long page = pages_s[page_ix(j) - pg0];
+        kreg[u] = *reinterpret_cast<const uint4v*>(p.k_cache + page * p.kb_stride + ((long long)page_off(j) * G + g) * D + dc * 8);
       }
     }
     // V: 8 groups of 4 keys; a 16-byte word = 2 value columns x 4 keys
@@ -282,8 +285,8 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
       const int j = kt * 32 + 4 * kg;
       vreg[u] = uint4v{0u, 0u, 0u, 0u};
       if (c < 8 * (DV / 2) && j <= j_hi) {
-        const long long page = pages_s[j / BS - pg0];
-        vreg[u] = *reinterpret_cast<const uint4v*>(p.v_cache + page * p.vb_stride + (long long)((j % BS) >> 2) * (4LL * G * DV) +
+        const long long page = pages_s[page_ix(j) - pg0];
+        vreg[u] = *reinterpret_cast<const uint4v*>(p.v_cache + page * p.vb_stride + (long long)(page_off(j) >> 2) * (4LL * G * DV) +
                                                    4LL * (g * DV + 2 * dc));
       }
     }
@@ -306,8 +309,10 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
       const int c = tid + 256 * u;
       if (c < 8 * (DV / 2)) {
         const int kg = c / (DV / 2), dc = c % (DV / 2);
-        *reinterpret_cast<uint2v*>(&Vt_s[(2 * dc) * kVPad + 4 * kg]) = uint2v{vreg[u][0], vreg[u][1]};
-        *reinterpret_cast<uint2v*>(&Vt_s[(2 * dc + 1) * kVPad + 4 * kg]) = uint2v{vreg[u][2], vreg[u][3]};
+        // key group kg (keys 4 kg ..) is k-slots 8 (kg & 3) + 4 (kg >> 2) ..: a lane group's 8 slots lie together
+        const int at = 8 * (kg & 3) + 4 * (kg >> 2);
+        *reinterpret_cast<uint2v*>(&Vt_s[(2 * dc) * kVPad + at]) = uint2v{vreg[u][0], vreg[u][1]};
+        *reinterpret_cast<uint2v*>(&Vt_s[(2 * dc + 1) * kVPad + at]) = uint2v{vreg[u][2], vreg[u][3]};
       }
     }
     if (tid < 96) bias_s[tid] = breg;
@@ -315,7 +320,7 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
 
   const int kt_lo = j_lo / 32, kt_hi = j_hi / 32;
   // the pages of keys [32 kt_lo, j_hi] once, so a tile's loads do not wait for a table lookup first
-  const int npg = j_hi / BS - pg0 + 1;
+  const int npg = page_ix(j_hi) - pg0 + 1;
   for (int c = tid; c < npg; c += 256) pages_s[c] = table[pg0 + c];
   __syncthreads();
   fetch(kt_lo);
@@ -395,10 +400,7 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
     }
 #pragma unroll
     for (int n = 0; n < NV; ++n) {
-      const bf16_t* vrow = &Vt_s[(n * 16 + r16) * kVPad];
-      const short4v b0 = *reinterpret_cast<const short4v*>(vrow + 4 * g4);
-      const short4v b1 = *reinterpret_cast<const short4v*>(vrow + 16 + 4 * g4);
-      const short8 b = short8{b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+      const short8 b = *reinterpret_cast<const short8*>(&Vt_s[(n * 16 + r16) * kVPad + 8 * g4]);
       O[n] = mfma16(ph, b, O[n]);
       O[n] = mfma16(pl, b, O[n]);
     }
@@ -442,10 +444,13 @@ extern "C" int r32_window_attn_mfma(const float* q, const void* k_cache, const v
                                     const float* bias, int window, void* out, int ldo, int H, int G, int D, int Dv,
                                     hipStream_t s) {
   if (n_items <= 0 || max_q <= 0) return 0;
-  if (!r32_window_attn_mfma_ok(D, Dv) || H % G != 0) return -1;
+  if (!r32_window_attn_mfma_ok(D, Dv) || H % G != 0 || (block_size & (block_size - 1)) != 0) return -1;
   WAttnMfmaParams p;
   p.q = q; p.k_cache = (const bf16_t*)k_cache; p.v_cache = (const bf16_t*)v_cache;
   p.kb_stride = kb_stride; p.vb_stride = vb_stride; p.block_size = block_size; p.positions = positions;
+  p.bs_shift = -1;
+  for (int b = 0; b < 20; ++b)
+    if ((1 << b) == block_size) p.bs_shift = b;
   p.cu_q = cu_q; p.k_lens = k_lens; p.tiles_per_item = (max_q + 63) / 64; p.block_tables = block_tables;
   p.bt_width = bt_width; p.bias = bias; p.window = window; p.out = (bf16_t*)out; p.ldo = ldo; p.H = H; p.G = G;
   const dim3 grid(n_items * p.tiles_per_item, H);

@@ -25,7 +25,7 @@ struct WAttnDecodeParams {
   const bf16_t* k_cache;
   const bf16_t* v_cache;
   long long kb_stride, vb_stride;
-  int block_size;
+  int block_size, bs_shift;  // block_size = 1 << bs_shift (the matrix-core kernels take power-of-two pages)
   const int* positions;    // [B]: the new token's position (its key is already in the cache)
   const int* block_tables;
   int bt_width;
@@ -49,7 +49,9 @@ __global__ void __launch_bounds__(64) window_attn_decode_kernel(const WAttnDecod
   const int base = (j_lo / 32) * 32 + split * p.keys_per_split;  // this split's first key (a multiple of 32)
   const int last = min(i, base + p.keys_per_split - 1);
   const int* table = p.block_tables + (size_t)b * p.bt_width;
-  const int BS = p.block_size;
+  const int BS = p.block_size, bsh = p.bs_shift;
+  auto page_ix = [&](int j) { return j >> bsh; };
+  auto page_off = [&](int j) { return j & (BS - 1); };
   const bool h_valid = r16 < nh;
   const int h = h0 + (h_valid ? r16 : 0);
 
@@ -77,7 +79,7 @@ __global__ void __launch_bounds__(64) window_attn_decode_kernel(const WAttnDecod
     for (int sub = 0; sub < 2; ++sub) {
       sacc[sub] = float4v{0.f, 0.f, 0.f, 0.f};
       const int j = min(t0 + sub * 16 + r16, i);  // (rows past the token are masked below: any valid row does)
-      const bf16_t* kr = p.k_cache + (long long)table[j / BS] * p.kb_stride + ((long long)(j % BS) * G + g) * D + 8 * g4;
+      const bf16_t* kr = p.k_cache + (long long)table[page_ix(j)] * p.kb_stride + ((long long)page_off(j) * G + g) * D + 8 * g4;
 #pragma unroll
       for (int kd = 0; kd < ND; ++kd) {
         const short8 a = *reinterpret_cast<const short8*>(kr + kd * 32);
@@ -123,8 +125,8 @@ __global__ void __launch_bounds__(64) window_attn_decode_kernel(const WAttnDecod
     // the lane's two 4-key groups: keys t0 + 4 g4 .. and t0 + 16 + 4 g4 .. (groups past the token: any valid one,
     // their weights are 0)
     const int ja = min(t0 + 4 * g4, (i / 4) * 4), jb = min(t0 + 16 + 4 * g4, (i / 4) * 4);
-    const bf16_t* va = p.v_cache + (long long)table[ja / BS] * p.vb_stride + (long long)((ja % BS) >> 2) * (4LL * G * DV) + 4LL * (g * DV + r16);
-    const bf16_t* vb = p.v_cache + (long long)table[jb / BS] * p.vb_stride + (long long)((jb % BS) >> 2) * (4LL * G * DV) + 4LL * (g * DV + r16);
+    const bf16_t* va = p.v_cache + (long long)table[page_ix(ja)] * p.vb_stride + (long long)(page_off(ja) >> 2) * (4LL * G * DV) + 4LL * (g * DV + r16);
+    const bf16_t* vb = p.v_cache + (long long)table[page_ix(jb)] * p.vb_stride + (long long)(page_off(jb) >> 2) * (4LL * G * DV) + 4LL * (g * DV + r16);
 #pragma unroll
     for (int n = 0; n < NV; ++n) {
 #pragma unroll
@@ -202,10 +204,13 @@ extern "C" int r32_window_attn_decode(const float* q, const void* k_cache, const
                                       int bt_width, const float* bias, int window, float* part_o, float* part_ml, int S,
                                       int max_keys, void* out, int ldo, int B, int H, int G, int D, int Dv, hipStream_t s) {
   if (B <= 0) return 0;
-  if (!r32_window_attn_mfma_ok(D, Dv) || H % G != 0 || S < 1) return -1;
+  if (!r32_window_attn_mfma_ok(D, Dv) || H % G != 0 || S < 1 || (block_size & (block_size - 1)) != 0) return -1;
   WAttnDecodeParams p;
   p.q = q; p.k_cache = (const bf16_t*)k_cache; p.v_cache = (const bf16_t*)v_cache; p.kb_stride = kb_stride;
   p.vb_stride = vb_stride; p.block_size = block_size; p.positions = positions; p.block_tables = block_tables;
+  p.bs_shift = -1;
+  for (int b = 0; b < 20; ++b)
+    if ((1 << b) == block_size) p.bs_shift = b;
   p.bt_width = bt_width; p.bias = bias; p.window = window; p.part_o = part_o; p.part_ml = part_ml; p.H = H; p.G = G;
   p.S = S;
   // a row's keys start at a multiple of 32 at or below its window's first key: up to max_keys + 31 keys to cover

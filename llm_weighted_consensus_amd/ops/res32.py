@@ -106,13 +106,14 @@ def window_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, p
     (it wants ``k_lens``, ``max_q`` and the ``bias`` table of :func:`distance_bias`) and decode rows on the
     split-key decode kernel (``bias``); everything else on the general kernel."""
     K = kernels()
-    if (cu_q is None and bias is not None and k_cache.dtype == torch.bfloat16 and positions.numel() > 0
-            and K.window_attn_mfma_ok(k_cache.shape[2] // G, v_cache.shape[2] // G)):
+    bs = k_cache.shape[1]
+    cores = (bias is not None and k_cache.dtype == torch.bfloat16 and bs & (bs - 1) == 0
+             and K.window_attn_mfma_ok(k_cache.shape[2] // G, v_cache.shape[2] // G))
+    if cores and cu_q is None and positions.numel() > 0:
         max_keys = min(int(window), block_tables.shape[1] * k_cache.shape[1])
         K.window_attn_decode(q, k_cache, v_cache, positions, block_tables, bias, int(window), max_keys, out, int(H), int(G))
         return out
-    if (cu_q is not None and k_lens is not None and bias is not None and max_q > 0 and k_cache.dtype == torch.bfloat16
-            and K.window_attn_mfma_ok(k_cache.shape[2] // G, v_cache.shape[2] // G)):
+    if cores and cu_q is not None and k_lens is not None and max_q > 0:
         K.window_attn_mfma(q, k_cache, v_cache, positions, cu_q, k_lens, int(max_q), block_tables, bias, int(window), out,
                            int(H), int(G))
         return out
