@@ -208,6 +208,7 @@ struct WAttnMfmaParams {
   int ldo, H, G;
 };
 
+constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kVPad = 40;  // keys per V^T row in LDS (32 + 8: rows stay 16-byte aligned, banks spread)
 
 template <int ND, int NV>
@@ -292,7 +293,7 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
     }
     if (tid < 96) {
       const int dist = pos0 - kt * 32 - 31 + tid;  // (row - key + 31) = tid
-      breg = dist >= 0 && dist < p.window ? bias_h[dist] : 0.f;
+      breg = dist >= 0 && dist < p.window ? bias_h[dist] * kLog2e : 0.f;  // the softmax runs in the log2 domain
     }
   };
   auto stash = [&](int buf) {
@@ -349,11 +350,11 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
     const bool inner = kt * 32 + 31 <= w_min && kt * 32 >= w_max - p.window + 1 && w_max - w_min == 15;
     float s[8];
     float mx = -1e30f;
+    const float* brow = bias_s + (qrow + 31 - 4 * g4);
     if (inner) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const int jl = (e >> 2) * 16 + 4 * g4 + (e & 3);
-        s[e] = sacc[e >> 2][e & 3] - bias_s[qrow - jl + 31];
+        s[e] = fmaf(sacc[e >> 2][e & 3], kLog2e, -brow[-((e >> 2) * 16 + (e & 3))]);
         mx = fmaxf(mx, s[e]);
       }
     } else {
@@ -362,19 +363,27 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
         const int jl = (e >> 2) * 16 + 4 * g4 + (e & 3);
         const int dist = i_q - (kt * 32 + jl);
         const bool ok = q_valid && dist >= 0 && dist < p.window;
-        s[e] = ok ? sacc[e >> 2][e & 3] - bias_s[qrow - jl + 31] : -1e30f;
+        s[e] = ok ? fmaf(sacc[e >> 2][e & 3], kLog2e, -brow[-((e >> 2) * 16 + (e & 3))]) : -1e30f;
         mx = fmaxf(mx, s[e]);
       }
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m, mx);
-    const float alpha = __expf(m - m_new);
+    const float alpha = __builtin_amdgcn_exp2f(m - m_new);
     float pe[8], psum = 0.f;
+    if (inner) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      pe[e] = s[e] > -1e29f ? __expf(s[e] - m_new) : 0.f;
-      psum += pe[e];
+      for (int e = 0; e < 8; ++e) {
+        pe[e] = __builtin_amdgcn_exp2f(s[e] - m_new);
+        psum += pe[e];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        pe[e] = s[e] > -1e29f ? __builtin_amdgcn_exp2f(s[e] - m_new) : 0.f;
+        psum += pe[e];
+      }
     }
     psum += __shfl_xor(psum, 16, 64);
     psum += __shfl_xor(psum, 32, 64);
