@@ -13,6 +13,7 @@ int r32_proj_norm_kv_write(const void*, int, const void*, const void*, const flo
                            int, hipStream_t);
 int r32_xielu(const void*, int, const void*, void*, int, int, int, int, hipStream_t);
 int r32_residual_add_scaled(float*, const void*, float, long long, int, hipStream_t);
+int r32_residual_add_partials(float*, const float*, int, float, long long, hipStream_t);
 int r32_window_attn(const float*, const void*, const void*, long long, long long, int, const int*, const int*, int,
                     const int*, int, const float*, const float*, int, void*, int, int, int, int, int, int, int,
                     hipStream_t);
@@ -147,6 +148,14 @@ void residual_add_scaled(Tensor x, Tensor y, double m) {
        "residual_add_scaled");
 }
 
+void residual_add_partials(Tensor x, Tensor parts, double m) {
+  want(x, torch::kFloat32, "residual_add_partials x");
+  want(parts, torch::kFloat32, "residual_add_partials parts");
+  TORCH_CHECK(parts.dim() >= 2 && parts.numel() == parts.size(0) * x.numel(), "residual_add_partials: parts [S, ...x]");
+  done(r32_residual_add_partials(x.data_ptr<float>(), parts.data_ptr<float>(), (int)parts.size(0), (float)m,
+                                 (long long)x.numel(), stream()), "residual_add_partials");
+}
+
 // q fp32 [T, H*D]; out [T, >= H*Dv] row-dense view of the cache dtype; block_tables [items, width] int32;
 // cu_q: int32 [items + 1] for prompt portions, absent when row t is item t.
 void window_attn(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, c10::optional<Tensor> cu_q,
@@ -259,6 +268,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("proj_norm_kv_write", &proj_norm_kv_write);
   m.def("xielu", &xielu);
   m.def("residual_add_scaled", &residual_add_scaled);
+  m.def("residual_add_partials", &residual_add_partials);
   m.def("window_attn", &window_attn);
   m.def("window_attn_mfma", &window_attn_mfma);
   m.def("window_attn_mfma_ok", &window_attn_mfma_ok);

@@ -10,7 +10,7 @@
 //                       cache; v (4-token interleaved in its pages) blended with the values of an earlier layer (v <- (1 - lam) v + lam v0) or
 //                       published as that v0, then into the paged cache
 //   xielu               z > 0: ap z^2 + z/2;  z <= 0: an (expm1(z) - z) + z/2, ap = softplus(p), an = 1/2 + softplus(q)
-//   residual_add_scaled x += m * y
+//   residual_add_scaled x += m * y          residual_add_partials x += m * sum_s y_s (fp32 split-K partials)
 #include "../common.h"
 
 namespace lwc {
@@ -156,6 +156,17 @@ __global__ void residual_add_scaled_kernel(float* __restrict__ x, const AT* __re
     x[e] += m * Elem<AT>::ld(y + e);
 }
 
+// x += m * sum_s parts[s]  (fp32 partial products of a split-K GEMM)
+__global__ void residual_add_partials_kernel(float* __restrict__ x, const float* __restrict__ parts, int S, float m,
+                                             long long total) {
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < total;
+       e += (long long)gridDim.x * blockDim.x) {
+    float acc = 0.f;
+    for (int s = 0; s < S; ++s) acc += parts[(long long)s * total + e];
+    x[e] += m * acc;
+  }
+}
+
 int grid_for(long long total, int block) {
   long long g = (total + block - 1) / block;
   return (int)(g < 1 ? 1 : (g > 65536 ? 65536 : g));
@@ -226,6 +237,12 @@ int r32_residual_add_scaled(float* x, const void* y, float m, long long total, i
   const int g = grid_for(total, 256);
   R32_DISPATCH(f32, (residual_add_scaled_kernel<bf16_t><<<g, 256, 0, s>>>(x, (const bf16_t*)y, m, total)),
                (residual_add_scaled_kernel<float><<<g, 256, 0, s>>>(x, (const float*)y, m, total)));
+  return (int)hipGetLastError();
+}
+
+int r32_residual_add_partials(float* x, const float* parts, int S, float m, long long total, hipStream_t s) {
+  if (total <= 0 || S <= 0) return 0;
+  residual_add_partials_kernel<<<grid_for(total, 256), 256, 0, s>>>(x, parts, S, m, total);
   return (int)hipGetLastError();
 }
 

@@ -90,6 +90,11 @@ def residual_add_scaled(x: torch.Tensor, y: torch.Tensor, m: float) -> None:
     kernels().residual_add_scaled(x, y, float(m))
 
 
+def residual_add_partials(x: torch.Tensor, parts: torch.Tensor, m: float) -> None:
+    """x (fp32) += m * parts.sum(0), parts fp32 [S, *x.shape] (the partial products of a split-K GEMM)."""
+    kernels().residual_add_partials(x, parts, float(m))
+
+
 def distance_bias(r1: torch.Tensor, r2: torch.Tensor, window: int) -> torch.Tensor:
     """The table b[h, n] = r1_h ln(1 + r2_h n), n < window (fp32), that the matrix-core kernel reads."""
     n = torch.arange(window, dtype=torch.float32, device=r1.device)

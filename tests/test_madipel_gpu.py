@@ -444,6 +444,20 @@ def test_generation_chunked_prefill_and_forks(gpu, tmp_path):
     assert eng.bm.num_free == eng.bm.num_blocks
 
 
+def test_split_reduction_output_projection(gpu, tmp_path):
+    """A model whose [o | down] reduction is long enough for the decode step's split-K path (few rows): decode rows
+    (split) and a long portion (one GEMM) both match the oracle."""
+    CONFIGS["wide"] = dict(width=32, vocab=288, layers=[dict(heads=2, kv_heads=1, dim=32, vdim=64, window=50, v_mix=True, ff=4096 - 128)])
+    cfg, W, model, eng = _build(tmp_path, "wide", torch.bfloat16, num_blocks=40, max_model_len=512)
+    assert model._split_ok
+    toks = _tokens(300, 288, 5)
+    ref = O.forward(cfg, W, toks)
+    got = [eng.step_tokens([("w", toks[:290], list(range(290)))])]
+    for i in range(290, 300):
+        got.append(eng.step_tokens([("w", [toks[i]], [0])], ["w"] if i == 299 else []))
+    assert _err(torch.cat(got), ref) < TOL[torch.bfloat16]
+
+
 def test_loader_refuses_wrong_shapes(gpu, tmp_path):
     from safetensors.torch import save_file
 
