@@ -167,6 +167,126 @@ __global__ void residual_add_partials_kernel(float* __restrict__ x, const float*
   }
 }
 
+// ---- 16-byte paths for bf16 activations (row widths, leading dimensions and bases multiples of 8 elements) ----
+constexpr int kMaxChunks = 8;  // 8-element chunks a thread keeps in registers (rows up to 256 * 8 * 8 elements)
+
+// LayerNorm of fp32 rows -> bf16: the row is read once (two float4 per chunk) and stays in registers.
+__global__ void __launch_bounds__(256)
+layernorm_f32_bf16x8_kernel(const float* __restrict__ x, const long long* __restrict__ rows, const bf16_t* __restrict__ w,
+                            const bf16_t* __restrict__ b, bf16_t* __restrict__ out, int d, float eps) {
+  __shared__ float scratch[16];
+  const size_t r = rows ? (size_t)rows[blockIdx.x] : (size_t)blockIdx.x;
+  const float* xr = x + r * d;
+  const int nch = d >> 3;
+  float v[kMaxChunks][8];
+  float s = 0.f;
+#pragma unroll
+  for (int u = 0; u < kMaxChunks; ++u) {
+    const int c = threadIdx.x + 256 * u;
+    if (c < nch) {
+      const float4v a0 = *reinterpret_cast<const float4v*>(xr + 8 * c), a1 = *reinterpret_cast<const float4v*>(xr + 8 * c + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[u][e] = a0[e];
+        v[u][4 + e] = a1[e];
+        s += a0[e] + a1[e];
+      }
+    }
+  }
+  const float mean = block_sum(s, scratch) / (float)d;
+  float q = 0.f;
+#pragma unroll
+  for (int u = 0; u < kMaxChunks; ++u) {
+    if (threadIdx.x + 256 * u < nch) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float c0 = v[u][e] - mean;
+        q += c0 * c0;
+      }
+    }
+  }
+  const float rstd = 1.0f / sqrtf(block_sum(q, scratch) / (float)d + eps);
+  bf16_t* o = out + (size_t)blockIdx.x * d;
+#pragma unroll
+  for (int u = 0; u < kMaxChunks; ++u) {
+    const int c = threadIdx.x + 256 * u;
+    if (c < nch) {
+      float wf[8], bf[8], y[8];
+      unpack8(*reinterpret_cast<const uint4v*>(w + 8 * c), wf);
+      unpack8(*reinterpret_cast<const uint4v*>(b + 8 * c), bf);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[e] = (v[u][e] - mean) * rstd * wf[e] + bf[e];
+      *reinterpret_cast<uint4v*>(o + 8 * c) = pack8(y);
+    }
+  }
+}
+
+// proj_norm_kv_write for bf16: the q | k | v part of the row is read once, 16 bytes per lane, and stays in registers.
+__global__ void __launch_bounds__(256)
+proj_norm_kv_write_bf16x8_kernel(const bf16_t* __restrict__ proj, int ldp, const bf16_t* __restrict__ wq,
+                                 const bf16_t* __restrict__ wk, const float* __restrict__ head_scale,
+                                 const bf16_t* __restrict__ lam_p, float* __restrict__ v0, int vmode,
+                                 const int* __restrict__ slots, float* __restrict__ q_out, bf16_t* __restrict__ k_cache,
+                                 bf16_t* __restrict__ v_cache, long long kb_stride, long long vb_stride, int block_size,
+                                 int H, int D, int nk, int nv, float eps) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  const int nq = H * D, cq = nq >> 3, ck = nk >> 3, cv = nv >> 3, nch = cq + ck + cv;
+  const bf16_t* pr = proj + (size_t)t * ldp;
+  float v[kMaxChunks][8];
+  float sq = 0.f, sk = 0.f;
+#pragma unroll
+  for (int u = 0; u < kMaxChunks; ++u) {
+    const int c = threadIdx.x + 256 * u;
+    if (c < nch) {
+      unpack8(*reinterpret_cast<const uint4v*>(pr + 8 * c), v[u]);
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += v[u][e] * v[u][e];
+      if (c < cq) sq += ss;
+      else if (c < cq + ck) sk += ss;
+    }
+  }
+  const float rq = 1.0f / sqrtf(block_sum(sq, scratch) / (float)nq + eps);
+  const float rk = 1.0f / sqrtf(block_sum(sk, scratch) / (float)nk + eps);
+  const int slot = slots[t];
+  const bool write = slot >= 0;
+  const long long blk = write ? slot / block_size : 0, off = write ? slot % block_size : 0;
+  const float lam = vmode == 2 ? bf2f(*lam_p) : 0.f;
+#pragma unroll
+  for (int u = 0; u < kMaxChunks; ++u) {
+    const int c = threadIdx.x + 256 * u;
+    if (c >= nch) continue;
+    if (c < cq) {
+      float wf[8];
+      unpack8(*reinterpret_cast<const uint4v*>(wq + 8 * c), wf);
+      const float hs = head_scale[(8 * c) / D] * rq;  // (D is a multiple of 8: a chunk lies in one head)
+      float* qo = q_out + (size_t)t * nq + 8 * c;
+      *reinterpret_cast<float4v*>(qo) = float4v{v[u][0] * hs * wf[0], v[u][1] * hs * wf[1], v[u][2] * hs * wf[2], v[u][3] * hs * wf[3]};
+      *reinterpret_cast<float4v*>(qo + 4) = float4v{v[u][4] * hs * wf[4], v[u][5] * hs * wf[5], v[u][6] * hs * wf[6], v[u][7] * hs * wf[7]};
+    } else if (c < cq + ck) {
+      if (write) {
+        const int i = 8 * (c - cq);
+        float wf[8], y[8];
+        unpack8(*reinterpret_cast<const uint4v*>(wk + i), wf);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) y[e] = v[u][e] * rk * wf[e];
+        *reinterpret_cast<uint4v*>(k_cache + blk * kb_stride + off * nk + i) = pack8(y);
+      }
+    } else {
+      const int i = 8 * (c - cq - ck);
+      bf16_t* vc = v_cache + blk * vb_stride + (off >> 2) * (4LL * nv) + (off & 3);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float x = v[u][e];
+        if (vmode == 1) v0[(size_t)t * nv + i + e] = x;
+        if (vmode == 2) x = (1.0f - lam) * x + lam * v0[(size_t)t * nv + i + e];
+        if (write) vc[4 * (i + e)] = f2bf(x);
+      }
+    }
+  }
+}
+
 int grid_for(long long total, int block) {
   long long g = (total + block - 1) / block;
   return (int)(g < 1 ? 1 : (g > 65536 ? 65536 : g));
@@ -196,6 +316,11 @@ int r32_embed_sinpos(const void* table, const int* tokens, const int* positions,
 int r32_layernorm(const float* x, const long long* rows, const void* w, const void* b, void* out, int T, int d,
                   float eps, int f32, hipStream_t s) {
   if (T <= 0) return 0;
+  if (!f32 && d % 8 == 0 && d <= 256 * 8 * kMaxChunks && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0 &&
+      ((uintptr_t)b & 15) == 0 && ((uintptr_t)out & 15) == 0) {
+    layernorm_f32_bf16x8_kernel<<<T, 256, 0, s>>>(x, rows, (const bf16_t*)w, (const bf16_t*)b, (bf16_t*)out, d, eps);
+    return (int)hipGetLastError();
+  }
   R32_DISPATCH(f32,
                (layernorm_f32_kernel<bf16_t><<<T, 256, 0, s>>>(x, rows, (const bf16_t*)w, (const bf16_t*)b, (bf16_t*)out, d, eps)),
                (layernorm_f32_kernel<float><<<T, 256, 0, s>>>(x, rows, (const float*)w, (const float*)b, (float*)out, d, eps)));
@@ -207,6 +332,14 @@ int r32_proj_norm_kv_write(const void* proj, int ldp, const void* wq, const void
                            void* v_cache, long long kb_stride, long long vb_stride, int block_size, int T, int H, int D,
                            int nk, int nv, float eps, int f32, hipStream_t s) {
   if (T <= 0) return 0;
+  if (!f32 && D % 8 == 0 && nk % 8 == 0 && nv % 8 == 0 && ldp % 8 == 0 && (H * D + nk + nv) <= 256 * 8 * kMaxChunks &&
+      kb_stride % 8 == 0 && ((uintptr_t)proj & 15) == 0 && ((uintptr_t)wq & 15) == 0 && ((uintptr_t)wk & 15) == 0 &&
+      ((uintptr_t)k_cache & 15) == 0 && ((uintptr_t)q_out & 15) == 0) {
+    proj_norm_kv_write_bf16x8_kernel<<<T, 256, 0, s>>>(
+        (const bf16_t*)proj, ldp, (const bf16_t*)wq, (const bf16_t*)wk, head_scale, (const bf16_t*)lam, v0, vmode, slots, q_out,
+        (bf16_t*)k_cache, (bf16_t*)v_cache, kb_stride, vb_stride, block_size, H, D, nk, nv, eps);
+    return (int)hipGetLastError();
+  }
   R32_DISPATCH(f32,
                (proj_norm_kv_write_kernel<bf16_t><<<T, 256, 0, s>>>(
                    (const bf16_t*)proj, ldp, (const bf16_t*)wq, (const bf16_t*)wk, head_scale, (const bf16_t*)lam, v0, vmode,

@@ -49,6 +49,11 @@ def test_layernorm_rows(gpu, dtype, tol):
     rows = torch.tensor([7, 0, 7, 3], device=gpu)
     out = res32.layernorm(x.to(gpu), _dev(w, dtype), _dev(b, dtype), 1e-3, rows=rows)
     assert (out.cpu().double() - ref[rows.cpu()]).abs().max() < tol * 4
+    # a width that is a multiple of 8 (the 16-byte path in bf16), more than one chunk per thread
+    x8, w8, b8 = torch.randn(5, 2312, generator=g) * 2 - 0.7, torch.randn(2312, generator=g).to(torch.bfloat16), torch.randn(2312, generator=g).to(torch.bfloat16)
+    ref8 = O.layer_norm(x8.double(), w8.double(), b8.double(), 1e-3)
+    out = res32.layernorm(x8.to(gpu), _dev(w8, dtype), _dev(b8, dtype), 1e-3, rows=torch.tensor([4, 1], device=gpu))
+    assert (out.cpu().double() - ref8[[4, 1]]).abs().max() < tol * 6
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 3e-2)])
@@ -101,7 +106,8 @@ def test_proj_norm_write_and_window_attention(gpu, dtype, tol, H, G, D, Dv, wind
     g = torch.Generator().manual_seed(H * 100 + D)
     n, bs, eps = 70, 16, 1e-4
     nq, nk, nv = H * D, G * D, G * Dv
-    proj = (torch.randn(n, nq + nk + nv + 5, generator=g) * 2).to(torch.bfloat16)
+    pad = 8 if D % 8 == 0 and Dv % 8 == 0 else 5  # (rows of 8-element multiples take the 16-byte path in bf16)
+    proj = (torch.randn(n, nq + nk + nv + pad, generator=g) * 2).to(torch.bfloat16)
     wq, wk = (1 + 0.3 * torch.randn(nq, generator=g)).to(torch.bfloat16), (1 + 0.3 * torch.randn(nk, generator=g)).to(torch.bfloat16)
     temp = (1 + torch.rand(H, generator=g)).to(torch.bfloat16)
     r1, r2 = (0.2 + torch.rand(H, generator=g)).to(torch.bfloat16), (0.2 + torch.rand(H, generator=g)).to(torch.bfloat16)
