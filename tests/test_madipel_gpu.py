@@ -464,6 +464,42 @@ def test_split_reduction_output_projection(gpu, tmp_path):
     assert _err(torch.cat(got), ref) < TOL[torch.bfloat16]
 
 
+def test_trace_replay_command_line(gpu, tmp_path):
+    """bin/trace_run as a user runs it: JSON lines in, ``done <step>`` lines and <step>.f32 files out; two sequences
+    interleaved (portions beside single tokens, one sitting a step out), pages given back at ``end``."""
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+    from safetensors.torch import save_file
+
+    c = CONFIGS["odd"]
+    cfg = O.make_config(c["width"], c["vocab"], c["layers"])
+    W = O.make_weights(cfg, 4)
+    mdir, out = tmp_path / "model", tmp_path / "out"
+    mdir.mkdir()
+    (mdir / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.contiguous() for k, v in W.items()}, str(mdir / "model.safetensors"))
+    a, b = _tokens(40, cfg["vocab"], 1), _tokens(21, cfg["vocab"], 2)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:30], "want": [0, 29]}], "end": []},
+             {"step": 1, "entries": [{"id": "b", "tokens": b[:20], "want": []}, {"id": "a", "tokens": a[30:31], "want": [0]}], "end": []},
+             {"step": 2, "entries": [{"id": "b", "tokens": b[20:], "want": [0]}], "end": ["b"]},
+             {"step": 3, "entries": [{"id": "a", "tokens": a[31:], "want": [8, 2]}], "end": ["a"]}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(mdir), "--dtype", "float32",
+                        "--out", str(out), "--max-tokens", "128"], input="\n".join(json.dumps(s) for s in steps) + "\n",
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [ln for ln in r.stdout.splitlines() if ln.startswith("done")] == [f"done {i}" for i in range(4)]
+    ra, rb = O.forward(cfg, W, a), O.forward(cfg, W, b)
+    want = {0: ra[[0, 29]], 2: rb[[20]], 3: ra[[39, 33]], 1: ra[[30]]}
+    for step, ref in want.items():
+        got = torch.from_numpy(np.fromfile(out / f"{step}.f32", dtype="<f4")).view(-1, cfg["vocab"])
+        assert _err(got, ref) < TOL[torch.float32]
+    assert sorted(os.listdir(out)) == ["0.f32", "1.f32", "2.f32", "3.f32"]
+
+
 def test_loader_refuses_wrong_shapes(gpu, tmp_path):
     from safetensors.torch import save_file
 
