@@ -52,6 +52,13 @@ __global__ void __launch_bounds__(64) window_attn_decode_kernel(const WAttnDecod
   const int BS = p.block_size, bsh = p.bs_shift;
   auto page_ix = [&](int j) { return j >> bsh; };
   auto page_off = [&](int j) { return j & (BS - 1); };
+  // the split's pages, one per lane, fetched once: a key's page then comes from a lane exchange instead of a table
+  // load that every K / V load would have to wait for (splits longer than 64 pages look the table up directly)
+  const int pg_base = page_ix(base);
+  const bool pages_in_lanes = page_ix(base + p.keys_per_split - 1) - pg_base < 64;
+  int my_page = 0;
+  if (pages_in_lanes && pg_base + lane <= page_ix(max(i, 0)) && base <= i) my_page = table[pg_base + lane];
+  auto page_of = [&](int j) { return pages_in_lanes ? __shfl(my_page, page_ix(j) - pg_base, 64) : table[page_ix(j)]; };
   const bool h_valid = r16 < nh;
   const int h = h0 + (h_valid ? r16 : 0);
 
@@ -79,7 +86,7 @@ __global__ void __launch_bounds__(64) window_attn_decode_kernel(const WAttnDecod
     for (int sub = 0; sub < 2; ++sub) {
       sacc[sub] = float4v{0.f, 0.f, 0.f, 0.f};
       const int j = min(t0 + sub * 16 + r16, i);  // (rows past the token are masked below: any valid row does)
-      const bf16_t* kr = p.k_cache + (long long)table[page_ix(j)] * p.kb_stride + ((long long)page_off(j) * G + g) * D + 8 * g4;
+      const bf16_t* kr = p.k_cache + (long long)page_of(j) * p.kb_stride + ((long long)page_off(j) * G + g) * D + 8 * g4;
 #pragma unroll
       for (int kd = 0; kd < ND; ++kd) {
         const short8 a = *reinterpret_cast<const short8*>(kr + kd * 32);
@@ -125,8 +132,8 @@ __global__ void __launch_bounds__(64) window_attn_decode_kernel(const WAttnDecod
     // the lane's two 4-key groups: keys t0 + 4 g4 .. and t0 + 16 + 4 g4 .. (groups past the token: any valid one,
     // their weights are 0)
     const int ja = min(t0 + 4 * g4, (i / 4) * 4), jb = min(t0 + 16 + 4 * g4, (i / 4) * 4);
-    const bf16_t* va = p.v_cache + (long long)table[page_ix(ja)] * p.vb_stride + (long long)(page_off(ja) >> 2) * (4LL * G * DV) + 4LL * (g * DV + r16);
-    const bf16_t* vb = p.v_cache + (long long)table[page_ix(jb)] * p.vb_stride + (long long)(page_off(jb) >> 2) * (4LL * G * DV) + 4LL * (g * DV + r16);
+    const bf16_t* va = p.v_cache + (long long)page_of(ja) * p.vb_stride + (long long)(page_off(ja) >> 2) * (4LL * G * DV) + 4LL * (g * DV + r16);
+    const bf16_t* vb = p.v_cache + (long long)page_of(jb) * p.vb_stride + (long long)(page_off(jb) >> 2) * (4LL * G * DV) + 4LL * (g * DV + r16);
 #pragma unroll
     for (int n = 0; n < NV; ++n) {
 #pragma unroll
