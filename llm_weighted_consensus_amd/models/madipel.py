@@ -240,26 +240,40 @@ class MadipelModel:
         return PagedLayerCache.elems_per_block(self._layer_dims(), block_size) * (4 if self.dtype == torch.float32 else 2)
 
     # ------------------------------------------------------------------ forward
-    def _forward(self, tokens, positions, slots, cache: PagedLayerCache, attend) -> torch.Tensor:
+    def _forward(self, tokens, positions, slots, cache: PagedLayerCache, attend, keep=None, keep_attend=None) -> torch.Tensor:
         """Every layer over the step's rows; ``attend(q, li, out)`` runs the attention of layer ``li`` into
-        ``out`` (a column slice).  Returns the fp32 residual stream [T, d]."""
+        ``out`` (a column slice).  Returns the fp32 residual stream [T, d].
+
+        ``keep`` (int64 rows; with ``keep_attend``, the attention over just those rows): only these rows' final
+        states are wanted (a prompt's last token, a few scored positions).  The LAST layer then still projects
+        q | k | v of every row and writes every row's keys and values (later steps read them), but runs the
+        attention, the feed-forward and the output projection on the kept rows only; returns [len(keep), d]."""
         cfg = self.cfg
         T = tokens.shape[0]
         x = res32.embed_sinpos(self.embed, tokens, positions, self.inv_freq)
         v0 = None
+        nl = len(self.layers)
         for li, (S, L) in enumerate(zip(cfg.layer_specs, self.layers)):
             m = S.mixer
+            no, nqkv = m.heads * m.vdim, m.nq + m.nk + m.nv
+            short = keep is not None and li + 1 == nl
             h = res32.layernorm(x, L.norm_w, L.norm_b, cfg.norm_eps)
-            proj = self._linear(h, L.w_in)
+            proj = self._linear(h, L.w_in[:nqkv] if short else L.w_in)
             if L.vmode and v0 is None:
                 v0 = torch.empty(T, m.nv, dtype=torch.float32, device=x.device)
             q = res32.proj_norm_kv_write(proj, L.q_norm, L.k_norm, L.head_scale, slots, cache.k[li], cache.v[li],
                                          m.heads, m.dim, cfg.norm_eps, lam=L.vmix, v0=v0, vmode=L.vmode)
-            no = m.heads * m.vdim
-            cat = torch.empty(T, no + S.ff, dtype=self.dtype, device=x.device)
-            attend(q, li, cat[:, :no])
-            if S.mlp_kind:
-                res32.xielu(proj[:, m.nq + m.nk + m.nv:], L.act, cat[:, no:])
+            if short:
+                x = x.index_select(0, keep)
+                cat = torch.empty(keep.numel(), no + S.ff, dtype=self.dtype, device=x.device)
+                keep_attend(q.index_select(0, keep), li, cat[:, :no])
+                if S.mlp_kind:
+                    res32.xielu(self._linear(h.index_select(0, keep), L.w_in[nqkv:]), L.act, cat[:, no:])
+            else:
+                cat = torch.empty(T, no + S.ff, dtype=self.dtype, device=x.device)
+                attend(q, li, cat[:, :no])
+                if S.mlp_kind:
+                    res32.xielu(proj[:, nqkv:], L.act, cat[:, no:])
             self._residual_linear(x, cat, L.w_out)
             if self.on_layer is not None:
                 self.on_layer(li, x)
@@ -311,8 +325,15 @@ class MadipelModel:
             if chk_run is not None:
                 chk_run(q, li, out, slice(n_dec, T))
 
-        x = self._forward(tokens, positions, slots, cache, attend)
-        return self._logits(x, logit_rows, float_logits)
+        # prompt portions of which few rows are wanted (a prompt's last token): the last layer on those rows only
+        keep = keep_attend = None
+        if n_dec == 0 and self.on_layer is None and 4 * logit_rows.numel() <= T:
+            keep = logit_rows
+            item = torch.bucketize(logit_rows, chunk["cu_q"][1:].to(torch.int64), right=True)
+            keep_attend = self._attend(cache, positions.index_select(0, logit_rows),
+                                       chunk["block_tables"].index_select(0, item))
+        x = self._forward(tokens, positions, slots, cache, attend, keep=keep, keep_attend=keep_attend)
+        return self._logits(x, None if keep is not None else logit_rows, float_logits)
 
     def prefill(self, tokens, positions, slots, cu_seqlens, max_seqlen, last_idx, cache, ctx=None):
         raise RuntimeError("Madipel prefills through forward_mixed over the paged cache (paged_prefill)")
