@@ -24,6 +24,28 @@ int r32_window_attn_mfma(const float*, const void*, const void*, long long, long
 int r32_window_attn_decode_splits(int, int, int, int);
 int r32_window_attn_decode(const float*, const void*, const void*, long long, long long, int, const int*, const int*, int,
                            const float*, int, float*, float*, int, int, void*, int, int, int, int, int, int, hipStream_t);
+int r32_conv_hist(const void*, int, const float*, const float*, long long, const int*, const int*, const int*, const int*,
+                  void*, int, void*, int, int, int, int, int, int, hipStream_t);
+int r32_conv_hist_update(const void*, int, float*, long long, const int*, const int*, int, int, int, int, hipStream_t);
+int r32_delta_rule_max_dim();
+int r32_delta_rule(const float*, int, const void*, int, int, int, const float*, const float*, float*, long long, const int*,
+                   const int*, const int*, float*, int, int, int, int, int, int, int, hipStream_t);
+int r32_head_norm_gate(const float*, int, const void*, int, const float*, void*, int, int, int, int, float, int, int,
+                       hipStream_t);
+int r32_embed_rows(const void*, const int*, float*, int, int, int, int, hipStream_t);
+int r32_head_norm_kv_write(const void*, int, int, int, const int*, const int*, float*, void*, void*, long long, long long,
+                           int, int, int, int, int, int, float, float, float, int, int, hipStream_t);
+int r32_gate_mul(void*, int, const void*, int, int, int, int, int, hipStream_t);
+int r32_gated_norm_residual(float*, const void*, int, const void*, int, const float*, void*, int, int, float, int, int,
+                            hipStream_t);
+int r32_rmsnorm_rows(const float*, const long long*, const float*, void*, int, int, float, int, hipStream_t);
+int r32_gelu_mul_rows(const void*, int, const void*, int, int, const int*, int, void*, int, int, int, hipStream_t);
+int r32_stack_mix(const float*, long long, const float*, int, float*, long long, hipStream_t);
+int r32_router_max_outputs();
+int r32_router(const float*, const float*, int, int, int, int, int*, float*, int*, int*, int*, int*, int*, int*, hipStream_t);
+int r32_expert_rows(const void*, int, const int*, const int*, const int*, int, const void*, const void*, float*, int, int,
+                    int, int, hipStream_t);
+int r32_moe_combine(const void*, int, const int*, const float*, const void*, int, int, int, float*, int, int, hipStream_t);
 }
 
 namespace {
@@ -40,6 +62,10 @@ int act_f32(const Tensor& t, const char* name) {
 
 void want(const Tensor& t, torch::ScalarType st, const char* name) {
   TORCH_CHECK(t.is_cuda() && t.scalar_type() == st && t.is_contiguous(), name, ": wrong device, dtype or layout");
+}
+
+void want_dev(const Tensor& t, torch::ScalarType st, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == st, name, ": wrong device or dtype");
 }
 
 void done(int rc, const char* name) { TORCH_CHECK(rc == 0, name, ": launch failed (", rc, ")"); }
@@ -259,6 +285,296 @@ void window_attn_decode(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positio
                               (int)max_keys, out.data_ptr(), ldo, B, (int)H, (int)G, D, Dv, stream()), "window_attn_decode");
 }
 
+
+// ---------------------------------------------------------------- recurrent state, gated layers, routed experts
+// Items: rows [cu[i], cu[i+1]) of one sequence at consecutive positions, with state slot item_slot[i].
+struct Items {
+  const int *row_item, *cu, *slot, *pos;
+  int T, n;
+};
+
+Items items_of(const Tensor& row_item, const Tensor& cu, const Tensor& item_slot, const Tensor& positions, int64_t slots,
+               const char* name) {
+  want(row_item, torch::kInt32, name);
+  want(cu, torch::kInt32, name);
+  want(item_slot, torch::kInt32, name);
+  want(positions, torch::kInt32, name);
+  const int T = (int)positions.numel(), n = (int)item_slot.numel();
+  TORCH_CHECK(row_item.numel() == T && cu.numel() == n + 1 && slots > 0, name, ": item tables disagree");
+  return {row_item.data_ptr<int>(), cu.data_ptr<int>(), item_slot.data_ptr<int>(), positions.data_ptr<int>(), T, n};
+}
+
+// hist fp32 [slots, taps - 1, C] (a strided view of a slot pool: slot stride taken from the view)
+long long hist_layout(const Tensor& hist, int taps, int C, const char* name) {
+  want_dev(hist, torch::kFloat32, name);
+  TORCH_CHECK(hist.dim() == 3 && hist.size(1) == taps - 1 && hist.size(2) == C && hist.stride(2) == 1 &&
+                  (taps == 1 || hist.stride(1) == C), name, ": history [slots, taps - 1, C]");
+  return (long long)hist.stride(0);
+}
+
+// mode 0: out = x + conv(x), out2 (optional) = x in out's dtype; mode 1: out = silu(conv(x)).  w fp32 [C, taps].
+void conv_hist(Tensor x, Tensor w, Tensor hist, Tensor row_item, Tensor cu, Tensor item_slot, Tensor positions, Tensor out,
+               c10::optional<Tensor> out2, int64_t mode) {
+  const int fi = act_f32(x, "conv_hist x"), fo = act_f32(out, "conv_hist out");
+  const int ldx = row_stride(x, "conv_hist x"), ldo = row_stride(out, "conv_hist out");
+  want(w, torch::kFloat32, "conv_hist w");
+  const int C = (int)x.size(1), taps = (int)w.size(1);
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == C && out.size(0) == x.size(0) && out.size(1) == C, "conv_hist: shapes disagree");
+  const long long ss = hist_layout(hist, taps, C, "conv_hist hist");
+  Items it = items_of(row_item, cu, item_slot, positions, hist.size(0), "conv_hist items");
+  TORCH_CHECK(it.T == x.size(0), "conv_hist: one position per row");
+  void* o2 = nullptr;
+  int ldo2 = 0;
+  if (out2.has_value()) {
+    TORCH_CHECK(mode == 0 && out2->scalar_type() == out.scalar_type() && out2->is_cuda() && out2->size(0) == x.size(0) &&
+                    out2->size(1) == C, "conv_hist: out2");
+    ldo2 = row_stride(*out2, "conv_hist out2");
+    o2 = out2->data_ptr();
+  }
+  done(r32_conv_hist(x.data_ptr(), ldx, w.data_ptr<float>(), hist.data_ptr<float>(), ss, it.row_item, it.cu, it.slot, it.pos,
+                     out.data_ptr(), ldo, o2, ldo2, it.T, C, taps, (int)mode, fi | (fo << 1), stream()), "conv_hist");
+}
+
+void conv_hist_update(Tensor x, Tensor hist, Tensor cu, Tensor item_slot, int64_t taps) {
+  const int fi = act_f32(x, "conv_hist_update x");
+  const int ldx = row_stride(x, "conv_hist_update x");
+  const int C = (int)x.size(1);
+  want(cu, torch::kInt32, "conv_hist_update cu");
+  want(item_slot, torch::kInt32, "conv_hist_update item_slot");
+  TORCH_CHECK(cu.numel() == item_slot.numel() + 1, "conv_hist_update: cu [items + 1]");
+  if (taps <= 1) return;
+  const long long ss = hist_layout(hist, (int)taps, C, "conv_hist_update hist");
+  done(r32_conv_hist_update(x.data_ptr(), ldx, hist.data_ptr<float>(), ss, cu.data_ptr<int>(), item_slot.data_ptr<int>(),
+                            (int)item_slot.numel(), C, (int)taps, fi, stream()), "conv_hist_update");
+}
+
+int64_t delta_rule_max_dim() { return r32_delta_rule_max_dim(); }
+
+// qkv fp32 [T, 2 G D + H Dv]; ba [T, ...] with beta logits at b_off and decay inputs at a_off (H columns each);
+// state fp32 [slots, H, D, Dv] view; out fp32 [T, H Dv]
+void delta_rule(Tensor qkv, Tensor ba, int64_t b_off, int64_t a_off, Tensor A_log, Tensor dt_bias, Tensor state, Tensor cu,
+                Tensor item_slot, Tensor positions, Tensor out, int64_t H, int64_t G) {
+  want_dev(qkv, torch::kFloat32, "delta_rule qkv");
+  const int ldq = row_stride(qkv, "delta_rule qkv");
+  const int f = act_f32(ba, "delta_rule ba");
+  const int ldb = row_stride(ba, "delta_rule ba");
+  want(A_log, torch::kFloat32, "delta_rule A_log");
+  want(dt_bias, torch::kFloat32, "delta_rule dt_bias");
+  want_dev(state, torch::kFloat32, "delta_rule state");
+  want(cu, torch::kInt32, "delta_rule cu");
+  want(item_slot, torch::kInt32, "delta_rule item_slot");
+  want(positions, torch::kInt32, "delta_rule positions");
+  want_dev(out, torch::kFloat32, "delta_rule out");
+  const int ldo = row_stride(out, "delta_rule out");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.stride(3) == 1 && state.stride(2) == state.size(3) &&
+                  state.stride(1) == state.size(2) * state.size(3), "delta_rule: state [slots, H, D, Dv]");
+  const int D = (int)state.size(2), Dv = (int)state.size(3), T = (int)qkv.size(0);
+  TORCH_CHECK(G > 0 && H % G == 0 && qkv.size(1) == 2 * G * D + H * Dv && out.size(0) == T && out.size(1) == H * Dv &&
+                  ba.size(0) == T && b_off >= 0 && a_off >= 0 && b_off + H <= ba.size(1) && a_off + H <= ba.size(1) &&
+                  A_log.numel() == H && dt_bias.numel() == H && positions.numel() == T && cu.numel() == item_slot.numel() + 1 &&
+                  D <= r32_delta_rule_max_dim(), "delta_rule: shapes disagree");
+  done(r32_delta_rule(qkv.data_ptr<float>(), ldq, ba.data_ptr(), ldb, (int)b_off, (int)a_off, A_log.data_ptr<float>(),
+                      dt_bias.data_ptr<float>(), state.data_ptr<float>(), (long long)state.stride(0), cu.data_ptr<int>(),
+                      item_slot.data_ptr<int>(), positions.data_ptr<int>(), out.data_ptr<float>(), ldo, (int)item_slot.numel(),
+                      (int)H, (int)G, D, Dv, f, stream()), "delta_rule");
+}
+
+// o fp32 [T, H Dv]; gate (mode 1 silu, 2 sigmoid; 0: unused) and out of the activation dtype; w fp32 [Dv] or absent
+void head_norm_gate(Tensor o, c10::optional<Tensor> gate, c10::optional<Tensor> w, Tensor out, int64_t H, double eps,
+                    int64_t mode) {
+  want_dev(o, torch::kFloat32, "head_norm_gate o");
+  const int ldi = row_stride(o, "head_norm_gate o"), ldo = row_stride(out, "head_norm_gate out");
+  const int f = act_f32(out, "head_norm_gate out");
+  const int T = (int)o.size(0);
+  TORCH_CHECK(H > 0 && o.size(1) % H == 0 && out.size(0) == T && out.size(1) == o.size(1), "head_norm_gate: shapes");
+  const int Dv = (int)(o.size(1) / H);
+  const void* gp = nullptr;
+  int ldg = 0;
+  if (mode != 0) {
+    TORCH_CHECK(gate.has_value() && gate->is_cuda() && gate->scalar_type() == out.scalar_type() && gate->size(0) == T &&
+                    gate->size(1) == o.size(1), "head_norm_gate: gate");
+    ldg = row_stride(*gate, "head_norm_gate gate");
+    gp = gate->data_ptr();
+  }
+  const float* wp = nullptr;
+  if (w.has_value()) {
+    want(*w, torch::kFloat32, "head_norm_gate w");
+    TORCH_CHECK(w->numel() == Dv, "head_norm_gate: w [Dv]");
+    wp = w->data_ptr<float>();
+  }
+  done(r32_head_norm_gate(o.data_ptr<float>(), ldi, gp, ldg, wp, out.data_ptr(), ldo, T, (int)H, Dv, (float)eps, (int)mode, f,
+                          stream()), "head_norm_gate");
+}
+
+void embed_rows(Tensor table, Tensor tokens, Tensor out) {
+  const int f = act_f32(table, "embed_rows table");
+  TORCH_CHECK(table.dim() == 2 && table.is_contiguous(), "embed_rows: table [V, d]");
+  want(tokens, torch::kInt32, "embed_rows tokens");
+  want(out, torch::kFloat32, "embed_rows out");
+  const int T = (int)tokens.numel(), d = (int)table.size(1);
+  TORCH_CHECK(out.numel() == (int64_t)T * d, "embed_rows: out [T, d]");
+  done(r32_embed_rows(table.data_ptr(), tokens.data_ptr<int>(), out.data_ptr<float>(), T, d, (int)table.size(0), f, stream()),
+       "embed_rows");
+}
+
+// proj [T, ...] row-dense: q at column 0 (H*D), k at k_off (G*D), values at v_off (G*Dv; v_off == k_off: the keys as
+// projected are the values)
+void head_norm_kv_write(Tensor proj, int64_t k_off, int64_t v_off, Tensor positions, Tensor slots, Tensor q_out,
+                        Tensor k_cache, Tensor v_cache, int64_t H, int64_t G, double eps, double scale, double coef,
+                        int64_t every) {
+  const int f = act_f32(proj, "head_norm_kv_write proj");
+  const int ldp = row_stride(proj, "head_norm_kv_write proj");
+  const int T = (int)proj.size(0);
+  want(positions, torch::kInt32, "head_norm_kv_write positions");
+  want(slots, torch::kInt32, "head_norm_kv_write slots");
+  want(q_out, torch::kFloat32, "head_norm_kv_write q_out");
+  TORCH_CHECK(k_cache.is_cuda() && v_cache.is_cuda() && k_cache.scalar_type() == proj.scalar_type() &&
+                  v_cache.scalar_type() == proj.scalar_type(), "head_norm_kv_write: caches of the activation dtype");
+  int NB, BS, nk, nv;
+  cache_layout(k_cache, v_cache, NB, BS, nk, nv, "head_norm_kv_write");
+  TORCH_CHECK(G > 0 && H > 0 && H % G == 0 && nk % G == 0 && nv % G == 0, "head_norm_kv_write: head counts");
+  const int D = nk / (int)G, Dv = nv / (int)G;
+  TORCH_CHECK(positions.numel() == T && slots.numel() == T && q_out.numel() == (int64_t)T * H * D && k_off >= H * D &&
+                  k_off + nk <= proj.size(1) && v_off >= 0 && v_off + nv <= proj.size(1) && every >= 0,
+              "head_norm_kv_write: shapes disagree");
+  done(r32_head_norm_kv_write(proj.data_ptr(), ldp, (int)k_off, (int)v_off, positions.data_ptr<int>(), slots.data_ptr<int>(),
+                              q_out.data_ptr<float>(), k_cache.data_ptr(), v_cache.data_ptr(), (long long)k_cache.stride(0),
+                              (long long)v_cache.stride(0), BS, T, (int)H, (int)G, D, Dv, (float)eps, (float)scale, (float)coef,
+                              (int)every, f, stream()), "head_norm_kv_write");
+}
+
+void gate_mul(Tensor a, Tensor g, int64_t mode) {
+  const int f = act_f32(a, "gate_mul a");
+  const int lda = row_stride(a, "gate_mul a"), ldg = row_stride(g, "gate_mul g");
+  TORCH_CHECK(g.is_cuda() && g.scalar_type() == a.scalar_type() && g.size(0) == a.size(0) && g.size(1) == a.size(1) &&
+                  (mode == 0 || mode == 1), "gate_mul: shapes or dtypes disagree");
+  done(r32_gate_mul(a.data_ptr(), lda, g.data_ptr(), ldg, (int)a.size(0), (int)a.size(1), (int)mode, f, stream()), "gate_mul");
+}
+
+void gated_norm_residual(Tensor x, Tensor y, c10::optional<Tensor> r, Tensor w, c10::optional<Tensor> x_cast, double eps) {
+  want(x, torch::kFloat32, "gated_norm_residual x");
+  want(w, torch::kFloat32, "gated_norm_residual w");
+  const int fy = act_f32(y, "gated_norm_residual y");
+  const int ldy = row_stride(y, "gated_norm_residual y");
+  const int T = (int)x.size(0), d = (int)x.size(1);
+  TORCH_CHECK(x.dim() == 2 && y.size(0) == T && y.size(1) == d && w.numel() == d, "gated_norm_residual: shapes disagree");
+  const void* rp = nullptr;
+  int ldr = 0, fr = 0;
+  if (r.has_value()) {
+    fr = act_f32(*r, "gated_norm_residual r");
+    ldr = row_stride(*r, "gated_norm_residual r");
+    TORCH_CHECK(r->size(0) == T && r->size(1) == d, "gated_norm_residual: gate logits [T, d]");
+    rp = r->data_ptr();
+  }
+  void* xc = nullptr;
+  if (x_cast.has_value()) {
+    want(*x_cast, torch::kBFloat16, "gated_norm_residual x_cast");
+    TORCH_CHECK(x_cast->numel() == x.numel(), "gated_norm_residual: x_cast [T, d]");
+    xc = x_cast->data_ptr();
+  }
+  done(r32_gated_norm_residual(x.data_ptr<float>(), y.data_ptr(), ldy, rp, ldr, w.data_ptr<float>(), xc, T, d, (float)eps, fy,
+                               fr, stream()), "gated_norm_residual");
+}
+
+void rmsnorm_rows(Tensor x, c10::optional<Tensor> rows, Tensor w, Tensor out, double eps) {
+  want(x, torch::kFloat32, "rmsnorm_rows x");
+  want(w, torch::kFloat32, "rmsnorm_rows w");
+  const int f = act_f32(out, "rmsnorm_rows out");
+  TORCH_CHECK(x.dim() == 2 && out.dim() == 2 && out.is_contiguous() && out.size(1) == x.size(1) && w.numel() == x.size(1),
+              "rmsnorm_rows: shapes disagree");
+  const long long* rp = nullptr;
+  if (rows.has_value()) {
+    want(*rows, torch::kInt64, "rmsnorm_rows rows");
+    TORCH_CHECK(rows->numel() == out.size(0), "rmsnorm_rows: one row index per output row");
+    rp = (const long long*)rows->data_ptr<int64_t>();
+  } else {
+    TORCH_CHECK(x.size(0) == out.size(0), "rmsnorm_rows: rows disagree");
+  }
+  done(r32_rmsnorm_rows(x.data_ptr<float>(), rp, w.data_ptr<float>(), out.data_ptr(), (int)out.size(0), (int)x.size(1),
+                        (float)eps, f, stream()), "rmsnorm_rows");
+}
+
+// out [T, n] = gelu_tanh(z [T, n]) * table[tokens[t]][off : off + n]
+void gelu_mul_rows(Tensor z, Tensor table, int64_t off, Tensor tokens, Tensor out) {
+  const int f = act_f32(z, "gelu_mul_rows z");
+  const int ldz = row_stride(z, "gelu_mul_rows z"), ldt = row_stride(table, "gelu_mul_rows table");
+  want(tokens, torch::kInt32, "gelu_mul_rows tokens");
+  const int T = (int)z.size(0), n = (int)z.size(1);
+  TORCH_CHECK(table.is_cuda() && table.scalar_type() == z.scalar_type() && out.is_cuda() && out.scalar_type() == z.scalar_type() &&
+                  out.is_contiguous() && out.dim() == 2 && out.size(0) == T && out.size(1) == n && tokens.numel() == T && off >= 0 &&
+                  off + n <= table.size(1), "gelu_mul_rows: shapes or dtypes disagree");
+  done(r32_gelu_mul_rows(z.data_ptr(), ldz, table.data_ptr(), ldt, (int)off, tokens.data_ptr<int>(), (int)table.size(0),
+                         out.data_ptr(), T, n, f, stream()), "gelu_mul_rows");
+}
+
+// out = sum_{j < n} coef[j] * X[j]; X fp32 [>= n, ...] contiguous, out one plane of it (it may be a plane of X
+// beyond the first n)
+void stack_mix(Tensor X, Tensor coef, int64_t n, Tensor out) {
+  want(X, torch::kFloat32, "stack_mix X");
+  want(coef, torch::kFloat32, "stack_mix coef");
+  want(out, torch::kFloat32, "stack_mix out");
+  TORCH_CHECK(X.dim() >= 2 && n >= 1 && n <= X.size(0) && coef.numel() >= n && out.numel() * X.size(0) == X.numel(),
+              "stack_mix: shapes disagree");
+  done(r32_stack_mix(X.data_ptr<float>(), (long long)out.numel(), coef.data_ptr<float>(), (int)n, out.data_ptr<float>(),
+                     (long long)out.numel(), stream()), "stack_mix");
+}
+
+int64_t router_max_outputs() { return r32_router_max_outputs(); }
+
+// z fp32 [T, NE] router logits, corr fp32 [NE]; the first E outputs are real experts.  Returns
+// (ids [T,k] i32, w [T,k] f32, row_off [E+1] i32, src [T*k] i32, row_expert [T*k] i32, inv [T*k] i32).
+std::vector<Tensor> router(Tensor z, Tensor corr, int64_t E, int64_t k) {
+  want(z, torch::kFloat32, "router z");
+  want(corr, torch::kFloat32, "router correction");
+  TORCH_CHECK(z.dim() == 2 && corr.numel() == z.size(1) && E >= 0 && E <= z.size(1) && k >= 1 && k <= z.size(1) &&
+                  z.size(1) <= r32_router_max_outputs(), "router: shapes disagree");
+  const int T = (int)z.size(0), NE = (int)z.size(1);
+  auto oi = z.options().dtype(torch::kInt32);
+  Tensor ids = torch::empty({T, k}, oi), w = torch::empty({T, k}, z.options()), rank = torch::empty({T, k}, oi);
+  Tensor counts = torch::zeros({std::max<int64_t>(E, 1)}, oi), row_off = torch::empty({E + 1}, oi);
+  Tensor src = torch::zeros({T * k}, oi), row_expert = torch::zeros({T * k}, oi), inv = torch::empty({T * k}, oi);
+  done(r32_router(z.data_ptr<float>(), corr.data_ptr<float>(), T, NE, (int)E, (int)k, ids.data_ptr<int>(), w.data_ptr<float>(),
+                  counts.data_ptr<int>(), rank.data_ptr<int>(), row_off.data_ptr<int>(), src.data_ptr<int>(),
+                  row_expert.data_ptr<int>(), inv.data_ptr<int>(), stream()), "router");
+  if (T == 0) row_off.zero_();
+  return {ids, w, row_off, src, row_expert, inv};
+}
+
+// h [T, d]; w_gu [E, 2 ff, d] (gate rows, then up rows), w_down [E, d, ff]; returns Y fp32 [len(src), d] (rows beyond
+// row_off[E] are not written)
+Tensor expert_rows(Tensor h, Tensor src, Tensor row_expert, Tensor row_off, Tensor w_gu, Tensor w_down) {
+  const int f = act_f32(h, "expert_rows h");
+  const int ldh = row_stride(h, "expert_rows h");
+  want(src, torch::kInt32, "expert_rows src");
+  want(row_expert, torch::kInt32, "expert_rows row_expert");
+  want(row_off, torch::kInt32, "expert_rows row_off");
+  const int d = (int)h.size(1);
+  TORCH_CHECK(w_gu.is_cuda() && w_down.is_cuda() && w_gu.is_contiguous() && w_down.is_contiguous() && w_gu.dim() == 3 &&
+                  w_down.dim() == 3 && w_gu.scalar_type() == h.scalar_type() && w_down.scalar_type() == h.scalar_type() &&
+                  w_gu.size(2) == d && w_down.size(1) == d && w_gu.size(1) == 2 * w_down.size(2) && w_gu.size(0) == w_down.size(0) &&
+                  row_off.numel() == w_gu.size(0) + 1 && row_expert.numel() == src.numel(), "expert_rows: shapes or dtypes disagree");
+  Tensor Y = torch::empty({src.numel(), d}, h.options().dtype(torch::kFloat32));
+  done(r32_expert_rows(h.data_ptr(), ldh, src.data_ptr<int>(), row_expert.data_ptr<int>(), row_off.data_ptr<int>(),
+                       (int)w_gu.size(0), w_gu.data_ptr(), w_down.data_ptr(), Y.data_ptr<float>(), (int)src.numel(), d,
+                       (int)w_down.size(2), f, stream()), "expert_rows");
+  return Y;
+}
+
+// out fp32 [T, d] = sum_j w[t][j] * (inv[t k + j] >= 0 ? Y[inv] : h[t])
+Tensor moe_combine(Tensor Y, Tensor inv, Tensor w, Tensor h) {
+  const int f = act_f32(h, "moe_combine h"), fy = act_f32(Y, "moe_combine Y");
+  const int ldh = row_stride(h, "moe_combine h");
+  want(inv, torch::kInt32, "moe_combine inv");
+  want(w, torch::kFloat32, "moe_combine w");
+  const int T = (int)h.size(0), d = (int)h.size(1);
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == T && inv.numel() == w.numel() && Y.is_contiguous() && Y.dim() == 2 && Y.size(1) == d,
+              "moe_combine: shapes disagree");
+  Tensor out = torch::empty({T, d}, h.options().dtype(torch::kFloat32));
+  done(r32_moe_combine(Y.data_ptr(), fy, inv.data_ptr<int>(), w.data_ptr<float>(), h.data_ptr(), ldh, T, (int)w.size(1),
+                       out.data_ptr<float>(), d, f, stream()), "moe_combine");
+  return out;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -273,4 +589,20 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("window_attn_mfma", &window_attn_mfma);
   m.def("window_attn_mfma_ok", &window_attn_mfma_ok);
   m.def("window_attn_decode", &window_attn_decode);
+  m.def("conv_hist", &conv_hist);
+  m.def("conv_hist_update", &conv_hist_update);
+  m.def("delta_rule", &delta_rule);
+  m.def("delta_rule_max_dim", &delta_rule_max_dim);
+  m.def("head_norm_gate", &head_norm_gate);
+  m.def("embed_rows", &embed_rows);
+  m.def("head_norm_kv_write", &head_norm_kv_write);
+  m.def("gate_mul", &gate_mul);
+  m.def("gated_norm_residual", &gated_norm_residual);
+  m.def("rmsnorm_rows", &rmsnorm_rows);
+  m.def("gelu_mul_rows", &gelu_mul_rows);
+  m.def("stack_mix", &stack_mix);
+  m.def("router", &router);
+  m.def("router_max_outputs", &router_max_outputs);
+  m.def("expert_rows", &expert_rows);
+  m.def("moe_combine", &moe_combine);
 }

@@ -1,0 +1,260 @@
+// Recurrent mechanisms with per-sequence state slots (gfx950, wave64).
+//
+// A step's rows are grouped in ITEMS: item i owns rows [cu[i], cu[i+1]) of one sequence, consecutive positions
+// (a decode row is an item of one row), and a state slot item_slot[i].  Nothing is read from a slot for a row
+// whose history lies before position 0, so a slot needs no clearing when it is handed to a new sequence.
+//
+//   conv_hist         causal convolution over time per channel, y_t = sum_s w[c][taps-1-s] x_(t-s), s < taps; the
+//                     inputs before the item's first row come from the slot's history (the last taps-1 inputs).
+//                     MODE 0: out = x + y (and optionally a cast copy of x); MODE 1: out = silu(y)
+//   conv_hist_update  the slot's history after the step: the last taps-1 inputs of old history ++ this step's rows
+//   delta_rule        gated delta rule, one wave per (item, head, 64 value columns), a state column per lane:
+//                       S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+//                     q, k made unit vectors per head (1e-6 inside the root), q times D^-1/2;
+//                     beta = sigmoid(b), g = exp(-exp(A_log) softplus(a + dt_bias)); state fp32 [slot][H][D][Dv]
+//   head_norm_gate    o / rms(o) over each head's Dv * w * silu(gate) (or sigmoid(gate), or no gate)
+#include "elem.h"
+
+namespace lwc {
+namespace {
+
+template <typename IT, typename OT, int MODE>
+__global__ void conv_hist_kernel(const IT* __restrict__ x, int ldx, const float* __restrict__ w,
+                                 const float* __restrict__ hist, long long slot_stride, const int* __restrict__ row_item,
+                                 const int* __restrict__ cu, const int* __restrict__ item_slot,
+                                 const int* __restrict__ positions, OT* __restrict__ out, int ldo, OT* __restrict__ out2,
+                                 int ldo2, int C, int taps) {
+  const int t = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int i = row_item[t];
+  const int r = t - cu[i], p = positions[t];
+  const float* h = hist + (long long)item_slot[i] * slot_stride;
+  const float cur = Elem<IT>::ld(x + (size_t)t * ldx + c);
+  float acc = w[(size_t)c * taps + taps - 1] * cur;
+  for (int s = 1; s < taps; ++s) {
+    float v = 0.f;
+    if (s <= r) v = Elem<IT>::ld(x + (size_t)(t - s) * ldx + c);
+    else if (s <= p) v = h[(size_t)(taps - 1 - (s - r)) * C + c];
+    acc += w[(size_t)c * taps + taps - 1 - s] * v;
+  }
+  if (MODE == 0) {
+    Elem<OT>::st(out + (size_t)t * ldo + c, cur + acc);
+    if (out2) Elem<OT>::st(out2 + (size_t)t * ldo2 + c, cur);
+  } else {
+    Elem<OT>::st(out + (size_t)t * ldo + c, silu_f(acc));
+  }
+}
+
+constexpr int kMaxTaps = 16;
+
+template <typename IT>
+__global__ void conv_hist_update_kernel(const IT* __restrict__ x, int ldx, float* __restrict__ hist, long long slot_stride,
+                                        const int* __restrict__ cu, const int* __restrict__ item_slot, int C, int taps) {
+  const int i = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int K = taps - 1, r0 = cu[i], n = cu[i + 1] - r0;
+  float* h = hist + (long long)item_slot[i] * slot_stride;
+  float old[kMaxTaps];
+#pragma unroll
+  for (int j = 0; j < kMaxTaps; ++j) old[j] = j < K ? h[(size_t)j * C + c] : 0.f;
+#pragma unroll
+  for (int j = 0; j < kMaxTaps; ++j) {
+    if (j < K) {
+      const int idx = n - K + j;
+      float v;
+      if (idx >= 0) {
+        v = Elem<IT>::ld(x + (size_t)(r0 + idx) * ldx + c);
+      } else {
+        v = 0.f;
+#pragma unroll
+        for (int m = 0; m < kMaxTaps; ++m) v = (m == j + n) ? old[m] : v;
+      }
+      h[(size_t)j * C + c] = v;
+    }
+  }
+}
+
+// qkv fp32 rows [q (G*D) | k (G*D) | v (H*Dv)]; ba rows hold the beta logits at column b_off and the decay
+// inputs at column a_off, one per head.
+template <typename AT, int DMAX>
+__global__ void __launch_bounds__(64) delta_rule_kernel(const float* __restrict__ qkv, int ldq, const AT* __restrict__ ba,
+                                                         int ldb, int b_off, int a_off, const float* __restrict__ A_log,
+                                                         const float* __restrict__ dt_bias, float* __restrict__ state,
+                                                         long long slot_stride, const int* __restrict__ cu,
+                                                         const int* __restrict__ item_slot,
+                                                         const int* __restrict__ positions, float* __restrict__ out,
+                                                         int ldo, int H, int G, int D, int Dv, int tiles) {
+  __shared__ float ks[DMAX], qs[DMAX];
+  const int lane = threadIdx.x;
+  const int item = blockIdx.y, h = blockIdx.x / tiles, tile = blockIdx.x - h * tiles;
+  const int col = tile * 64 + lane;
+  const bool live = col < Dv;
+  const int kvh = h / (H / G);
+  const int r0 = cu[item], r1 = cu[item + 1];
+  if (r1 <= r0) return;
+  float* Sg = state + (long long)item_slot[item] * slot_stride + ((size_t)h * D) * Dv + col;
+  float S[DMAX];
+  const bool fresh = positions[r0] == 0;
+#pragma unroll
+  for (int i = 0; i < DMAX; ++i) S[i] = (i < D && live && !fresh) ? Sg[(size_t)i * Dv] : 0.f;
+  const float nA = -expf(A_log[h]), dtb = dt_bias[h];
+  const float qscale = 1.0f / sqrtf((float)D);
+  const int nq = G * D;
+  for (int row = r0; row < r1; ++row) {
+    const float* qr = qkv + (size_t)row * ldq + kvh * D;
+    const float* kr = qr + nq;
+    float sq = 0.f, sk = 0.f;
+    for (int i = lane; i < D; i += 64) {
+      const float a = qr[i], b = kr[i];
+      sq += a * a;
+      sk += b * b;
+    }
+    sq = wave_sum(sq);
+    sk = wave_sum(sk);
+    const float rq = qscale / sqrtf(sq + 1e-6f), rk = 1.0f / sqrtf(sk + 1e-6f);
+    __syncthreads();
+    for (int i = lane; i < D; i += 64) {
+      qs[i] = qr[i] * rq;
+      ks[i] = kr[i] * rk;
+    }
+    __syncthreads();
+    const float v = live ? qkv[(size_t)row * ldq + 2 * nq + h * Dv + col] : 0.f;
+    const float beta = sigmoid_f(Elem<AT>::ld(ba + (size_t)row * ldb + b_off + h));
+    const float g = expf(nA * softplus_f(Elem<AT>::ld(ba + (size_t)row * ldb + a_off + h) + dtb));
+    float dot = 0.f;
+#pragma unroll
+    for (int i = 0; i < DMAX; ++i)
+      if (i < D) {
+        S[i] *= g;
+        dot += S[i] * ks[i];
+      }
+    const float u = beta * (v - dot);
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < DMAX; ++i)
+      if (i < D) {
+        S[i] += ks[i] * u;
+        o += S[i] * qs[i];
+      }
+    if (live) out[(size_t)row * ldo + h * Dv + col] = o;
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < DMAX; ++i)
+      if (i < D) Sg[(size_t)i * Dv] = S[i];
+  }
+}
+
+// GATE 0: none, 1: silu(gate), 2: sigmoid(gate)
+template <typename AT, int GATE>
+__global__ void head_norm_gate_kernel(const float* __restrict__ o, int ldi, const AT* __restrict__ gate, int ldg,
+                                      const float* __restrict__ w, AT* __restrict__ out, int ldo, int H, int Dv,
+                                      float eps) {
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  for (int h = wv; h < H; h += nw) {
+    const float* oh = o + (size_t)t * ldi + h * Dv;
+    float s = 0.f;
+    for (int i = lane; i < Dv; i += 64) s += oh[i] * oh[i];
+    const float rstd = 1.0f / sqrtf(wave_sum(s) / (float)Dv + eps);
+    for (int i = lane; i < Dv; i += 64) {
+      float y = oh[i] * rstd * (w ? w[i] : 1.0f);
+      if (GATE) {
+        const float z = Elem<AT>::ld(gate + (size_t)t * ldg + h * Dv + i);
+        y *= GATE == 1 ? silu_f(z) : sigmoid_f(z);
+      }
+      Elem<AT>::st(out + (size_t)t * ldo + h * Dv + i, y);
+    }
+  }
+}
+
+}  // namespace
+}  // namespace lwc
+
+using namespace lwc;
+
+// io: bit 0 = input fp32 (else bf16), bit 1 = output fp32 (else bf16)
+extern "C" int r32_conv_hist(const void* x, int ldx, const float* w, const float* hist, long long slot_stride,
+                             const int* row_item, const int* cu, const int* item_slot, const int* positions, void* out,
+                             int ldo, void* out2, int ldo2, int T, int C, int taps, int mode, int io, hipStream_t s) {
+  if (T <= 0 || C <= 0) return 0;
+  if (taps < 1 || taps > kMaxTaps) return -1;
+  dim3 grid((C + 255) / 256, T);
+#define LWC_CONV(IT, OT, M)                                                                                          \
+  conv_hist_kernel<IT, OT, M><<<grid, 256, 0, s>>>((const IT*)x, ldx, w, hist, slot_stride, row_item, cu, item_slot, \
+                                                   positions, (OT*)out, ldo, (OT*)out2, ldo2, C, taps)
+  if (mode == 0) {
+    if (io == 3) LWC_CONV(float, float, 0);
+    else if (io == 1) LWC_CONV(float, bf16_t, 0);
+    else if (io == 0) LWC_CONV(bf16_t, bf16_t, 0);
+    else return -1;
+  } else {
+    if (io == 3) LWC_CONV(float, float, 1);
+    else if (io == 2) LWC_CONV(bf16_t, float, 1);
+    else if (io == 0) LWC_CONV(bf16_t, bf16_t, 1);
+    else return -1;
+  }
+#undef LWC_CONV
+  LWC_CHECK_LAUNCH();
+  return 0;
+}
+
+extern "C" int r32_conv_hist_update(const void* x, int ldx, float* hist, long long slot_stride, const int* cu,
+                                    const int* item_slot, int items, int C, int taps, int in_f32, hipStream_t s) {
+  if (items <= 0 || C <= 0 || taps <= 1) return 0;
+  if (taps > kMaxTaps) return -1;
+  dim3 grid((C + 255) / 256, items);
+  if (in_f32) conv_hist_update_kernel<float><<<grid, 256, 0, s>>>((const float*)x, ldx, hist, slot_stride, cu, item_slot, C, taps);
+  else conv_hist_update_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)x, ldx, hist, slot_stride, cu, item_slot, C, taps);
+  LWC_CHECK_LAUNCH();
+  return 0;
+}
+
+extern "C" int r32_delta_rule_max_dim() { return 256; }
+
+extern "C" int r32_delta_rule(const float* qkv, int ldq, const void* ba, int ldb, int b_off, int a_off, const float* A_log,
+                              const float* dt_bias, float* state, long long slot_stride, const int* cu,
+                              const int* item_slot, const int* positions, float* out, int ldo, int items, int H, int G,
+                              int D, int Dv, int f32, hipStream_t s) {
+  if (items <= 0) return 0;
+  if (D < 1 || D > 256 || H % G != 0) return -1;
+  const int tiles = (Dv + 63) / 64;
+  dim3 grid(H * tiles, items);
+#define LWC_DELTA(AT, DM)                                                                                              \
+  delta_rule_kernel<AT, DM><<<grid, 64, 0, s>>>(qkv, ldq, (const AT*)ba, ldb, b_off, a_off, A_log, dt_bias, state,    \
+                                                slot_stride, cu, item_slot, positions, out, ldo, H, G, D, Dv, tiles)
+  if (f32) {
+    if (D <= 64) LWC_DELTA(float, 64);
+    else if (D <= 128) LWC_DELTA(float, 128);
+    else LWC_DELTA(float, 256);
+  } else {
+    if (D <= 64) LWC_DELTA(bf16_t, 64);
+    else if (D <= 128) LWC_DELTA(bf16_t, 128);
+    else LWC_DELTA(bf16_t, 256);
+  }
+#undef LWC_DELTA
+  LWC_CHECK_LAUNCH();
+  return 0;
+}
+
+extern "C" int r32_head_norm_gate(const float* o, int ldi, const void* gate, int ldg, const float* w, void* out, int ldo,
+                                  int T, int H, int Dv, float eps, int gate_mode, int f32, hipStream_t s) {
+  if (T <= 0) return 0;
+  const int threads = H >= 4 ? 256 : 64 * H;
+#define LWC_HNG(AT, GM)                                                                                           \
+  head_norm_gate_kernel<AT, GM><<<T, threads, 0, s>>>(o, ldi, (const AT*)gate, ldg, w, (AT*)out, ldo, H, Dv, eps)
+  if (f32) {
+    if (gate_mode == 0) LWC_HNG(float, 0);
+    else if (gate_mode == 1) LWC_HNG(float, 1);
+    else LWC_HNG(float, 2);
+  } else {
+    if (gate_mode == 0) LWC_HNG(bf16_t, 0);
+    else if (gate_mode == 1) LWC_HNG(bf16_t, 1);
+    else LWC_HNG(bf16_t, 2);
+  }
+#undef LWC_HNG
+  LWC_CHECK_LAUNCH();
+  return 0;
+}

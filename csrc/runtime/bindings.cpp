@@ -135,7 +135,7 @@ PYBIND11_MODULE(_runtime, m) {
       .def("blocks_for", &BlockManager::blocks_for)
       .def("can_allocate", &BlockManager::can_allocate)
       .def("add_sequence", &BlockManager::add_sequence)
-      .def("fork", &BlockManager::fork)
+      .def("fork", &BlockManager::fork, py::arg("parent"), py::arg("child"), py::arg("take_state") = false)
       .def("append_token", &BlockManager::append_token)
       .def("append_cost", &BlockManager::append_cost)
       .def("free_sequence", &BlockManager::free_sequence)
@@ -151,6 +151,11 @@ PYBIND11_MODULE(_runtime, m) {
       .def("slot", &BlockManager::slot)
       .def("refcount", &BlockManager::refcount)
       .def("take_copies", &BlockManager::take_copies)
+      .def("set_state_slots", &BlockManager::set_state_slots)
+      .def_property_readonly("num_state_slots", &BlockManager::num_state_slots)
+      .def_property_readonly("num_free_state_slots", &BlockManager::num_free_state_slots)
+      .def("state_slot", &BlockManager::state_slot)
+      .def("take_state_copies", &BlockManager::take_state_copies)
       .def("append_cost_total", &BlockManager::append_cost_total)
       .def("swap_out",
            [](BlockManager& bm, const std::vector<int64_t>& seqs) {

@@ -129,6 +129,7 @@ int64_t BlockManager::add_sequence_cached(int64_t seq, const std::vector<int32_t
   for (int32_t b : hit) in_lru += ref_[b] == 0;
   if (num_free() - in_lru < need) throw std::runtime_error("BlockManager: out of KV blocks");
   Seq s;
+  s.state = alloc_state();
   s.blocks.reserve(blocks_for(n) + 8);
   for (int32_t b : hit) {
     acquire_cached(b);
@@ -168,16 +169,25 @@ void BlockManager::add_sequence(int64_t seq, int64_t num_tokens) {
   const int need = blocks_for(num_tokens);
   if (!can_allocate(need)) throw std::runtime_error("BlockManager: out of KV blocks");
   Seq s;
+  s.state = alloc_state();
   s.blocks.reserve(need + 8);
   for (int i = 0; i < need; ++i) s.blocks.push_back(alloc_block());
   s.len = num_tokens;
   seqs_.emplace(seq, std::move(s));
 }
 
-void BlockManager::fork(int64_t parent, int64_t child) {
+void BlockManager::fork(int64_t parent, int64_t child, bool take_state) {
   if (seqs_.count(child)) throw std::invalid_argument("BlockManager: sequence exists " + std::to_string(child));
-  const Seq& p = get(parent);
+  Seq& p = get(parent);
   Seq c;
+  if (take_state && p.state >= 0) {  // the parent is about to be freed: its slot goes on with this child
+    c.state = p.state;
+    p.state = -1;
+  } else {
+    if (state_slots_ > 0 && p.state < 0) throw std::logic_error("BlockManager: fork of a sequence that gave its state away");
+    c.state = alloc_state();
+    if (c.state >= 0) state_copies_.emplace_back(p.state, c.state);
+  }
   c.blocks = p.blocks;
   c.len = p.len;
   for (int32_t b : c.blocks) ++ref_[b];
@@ -218,6 +228,7 @@ void BlockManager::free_sequence(int64_t seq) {
   auto it = seqs_.find(seq);
   if (it == seqs_.end()) return;
   for (int32_t b : it->second.blocks) release(b);
+  release_state(it->second.state);
   seqs_.erase(it);
 }
 
@@ -263,6 +274,8 @@ std::vector<int32_t> BlockManager::swap_in(const std::vector<int64_t>& seqs, int
       if (x < 0 || x >= n) throw std::out_of_range("BlockManager::swap_in: block index out of range");
   }
   if (!can_allocate(n)) throw std::runtime_error("BlockManager: out of KV blocks");
+  if (state_slots_ > 0 && state_free_.size() < seqs.size())
+    throw std::runtime_error("BlockManager: out of recurrent-state slots");
   std::vector<int32_t> phys(n);
   for (int i = 0; i < n; ++i) phys[i] = alloc_block();  // refcount 1 each
   std::vector<int32_t> refs(n, 0);
@@ -280,9 +293,37 @@ std::vector<int32_t> BlockManager::swap_in(const std::vector<int64_t>& seqs, int
     s.blocks.reserve(tables[i].size() + 8);
     for (int32_t x : tables[i]) s.blocks.push_back(phys[x]);
     s.len = lens[i];
+    s.state = alloc_state();
     seqs_.emplace(seqs[i], std::move(s));
   }
   return phys;
+}
+
+void BlockManager::set_state_slots(int n) {
+  if (!seqs_.empty()) throw std::logic_error("BlockManager: set_state_slots while sequences exist");
+  if (n < 0) throw std::invalid_argument("BlockManager: negative number of state slots");
+  state_slots_ = n;
+  state_free_.clear();
+  for (int s = n - 1; s >= 0; --s) state_free_.push_back(s);
+  state_copies_.clear();
+}
+
+int32_t BlockManager::alloc_state() {
+  if (state_slots_ == 0) return -1;
+  if (state_free_.empty()) throw std::runtime_error("BlockManager: out of recurrent-state slots");
+  const int32_t s = state_free_.back();
+  state_free_.pop_back();
+  return s;
+}
+
+void BlockManager::release_state(int32_t slot) {
+  if (slot >= 0) state_free_.push_back(slot);
+}
+
+std::vector<std::pair<int32_t, int32_t>> BlockManager::take_state_copies() {
+  std::vector<std::pair<int32_t, int32_t>> out;
+  out.swap(state_copies_);
+  return out;
 }
 
 std::vector<std::pair<int32_t, int32_t>> BlockManager::take_copies() {

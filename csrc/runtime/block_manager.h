@@ -35,7 +35,7 @@ class BlockManager {
   // Allocate a new sequence able to hold `num_tokens` tokens (its length is set to num_tokens).
   void add_sequence(int64_t seq, int64_t num_tokens);
   // Child shares every block of the parent (refcount++), same length.
-  void fork(int64_t parent, int64_t child);
+  void fork(int64_t parent, int64_t child, bool take_state = false);
   // Grow the sequence by one token; returns the cache slot (block*BS + offset) of that token.
   // Allocates a new block at block boundaries and performs copy-on-write on a shared last block.
   int64_t append_token(int64_t seq);
@@ -71,6 +71,17 @@ class BlockManager {
   // Copy-on-write copies queued since the last call (src, dst); cleared by this call.
   std::vector<std::pair<int32_t, int32_t>> take_copies();
 
+  // Recurrent-state slots for models whose layers carry per-sequence state besides keys and values (a running
+  // matrix, the last inputs of a convolution): with n > 0 every sequence holds exactly one of n slots from
+  // add_sequence / fork / swap_in until free_sequence (swap_out frees it too: the caller saves the slot's
+  // contents first).  A fork queues a (parent slot, child slot) copy for the caller to carry out on the device.
+  // Only while no sequence exists.
+  void set_state_slots(int n);
+  int num_state_slots() const { return state_slots_; }
+  int num_free_state_slots() const { return (int)state_free_.size(); }
+  int32_t state_slot(int64_t seq) const { return get(seq).state; }
+  std::vector<std::pair<int32_t, int32_t>> take_state_copies();
+
   // ---- automatic prefix caching (cross-request KV reuse) ----
   // A FULL prompt block can be registered under a chain key: key_i = H(key_{i-1}, the block's BS token
   // ids), key_{-1} = a root constant, so a key names the whole token prefix up to that block.  A later
@@ -94,7 +105,10 @@ class BlockManager {
   struct Seq {
     std::vector<int32_t> blocks;
     int64_t len = 0;
+    int32_t state = -1;  // recurrent-state slot (set_state_slots), -1 without
   };
+  int32_t alloc_state();
+  void release_state(int32_t slot);
   const Seq& get(int64_t seq) const;
   Seq& get(int64_t seq);
   int32_t alloc_block();
@@ -118,6 +132,9 @@ class BlockManager {
   std::vector<std::list<int32_t>::iterator> lru_pos_;
   std::unordered_map<int64_t, Seq> seqs_;
   std::vector<std::pair<int32_t, int32_t>> copies_;
+  int state_slots_ = 0;
+  std::vector<int32_t> state_free_;
+  std::vector<std::pair<int32_t, int32_t>> state_copies_;
 };
 
 }  // namespace lwc

@@ -112,7 +112,7 @@ def build_res32(jobs: int = 8, force: bool = False) -> Path:
     kdir = CSRC / "kernels" / "res32"
     obj_dir = BUILD / "res32"
     obj_dir.mkdir(parents=True, exist_ok=True)
-    headers = sorted((CSRC / "kernels").glob("*.h"))
+    headers = sorted((CSRC / "kernels").glob("*.h")) + sorted(kdir.glob("*.h"))
     base = ["hipcc", f"--offload-arch={ARCH}", "-O3", "-fPIC", "-std=c++17", "-Wno-unused-result", *NO_PACKED_FP32,
             f"-I{kdir}"]
     tflags, tlibs = _torch_flags("_res32")

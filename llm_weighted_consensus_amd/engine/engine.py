@@ -149,7 +149,7 @@ class _GraphBucket:
         self.graph_logits: Dict[bool, torch.Tensor] = {}
         self.pool = None
         segs: List[Tuple[str, int]] = [("block_tables", B * width), ("ctx_lens", B), ("slots", B), ("positions", B),
-                                       ("tokens", B), ("tiles", max(1, max_tiles) * 3)]
+                                       ("tokens", B), ("state_slots", B), ("tiles", max(1, max_tiles) * 3)]
         segs += [(n, B) for n in _F32_PARAMS + _I32_PARAMS]
         segs += [("seeds", 2 * B), ("offsets", 2 * B)]
         self.off: Dict[str, Tuple[int, int]] = {}
@@ -326,6 +326,7 @@ class _SwapRecord:
     tables: List[List[int]]     # per sequence: indices into the n saved blocks
     lens: List[int]
     event: Optional[torch.cuda.Event]
+    state: Optional[torch.Tensor] = None  # the sequences' recurrent-state slots [len(seqs), slot_elems], host
 
 
 class LLMEngine:
@@ -363,6 +364,14 @@ class LLMEngine:
         self.cache = (model.new_cache(num_blocks, block_size) if hasattr(model, "new_cache")
                       else KVCache(self.cfg, num_blocks, block_size, self.device))
         self.bm = BlockManager(num_blocks, block_size)
+        # models with recurrent layers: one state slot per live sequence, handed out by the block manager with the
+        # sequence's blocks (models/state.py); the pool's last slot is scratch for padded rows and warm-up runs
+        self.state = None
+        if getattr(model, "has_state", False):
+            if prefix_caching:
+                raise ValueError("prefix caching cannot skip a prompt's head for a model with recurrent state")
+            self.state = model.new_state(max_batch)
+            self.bm.set_state_slots(max_batch)
         # cross-request prefix cache (C++ block manager): prompts that start with an already computed
         # token prefix (the shared messages of a score request's voters, a repeated conversation) reuse
         # its full KV blocks and prefill only the tail
@@ -430,6 +439,10 @@ class LLMEngine:
         if len(prompt_ids) + params.max_tokens > self.max_model_len:
             raise ValueError(f"prompt ({len(prompt_ids)}) + max_tokens ({params.max_tokens}) exceeds "
                              f"max_model_len ({self.max_model_len})")
+        if prefilled is not None and self.state is not None:
+            raise ValueError("a prompt prefilled elsewhere brings no recurrent state")
+        if self.state is not None and n > self.max_batch:
+            raise ValueError("n exceeds the number of recurrent-state slots (max_batch)")
         g = SequenceGroup(self, list(prompt_ids), params, n, callback)
         g.prefilled = prefilled
         if isinstance(ctx, dict):
@@ -568,7 +581,8 @@ class LLMEngine:
         logits = self.model.forward_mixed(_h2d(toks_all, torch.int32, dev), _h2d(pos, torch.int32, dev),
                                           _h2d(np.concatenate(slot_parts), torch.int32, dev), self.cache, B, dec_in,
                                           chunk_in, _h2d(rows or [0], torch.int64, dev),
-                                          **({"float_logits": True} if getattr(self.model, "float_logits", False) else {}))
+                                          **({"float_logits": True} if getattr(self.model, "float_logits", False) else {}),
+                                          **self._state_args([sid for _, sid, _, _ in dec + por]))
         if rows:
             out = logits.float()
         self.stats["prefill_tokens"] += len(toks_all) - B
@@ -578,6 +592,28 @@ class LLMEngine:
             if sid is not None:
                 bm.free_sequence(sid)
         return out
+
+    # ------------------------------------------------------------------ recurrent state
+    def _state_args(self, sids) -> dict:
+        """The model's extra arguments for a step over the block-manager sequences ``sids`` (decode rows first, then
+        portions): the state pool and every sequence's slot.  Empty for models without recurrent state."""
+        if self.state is None:
+            return {}
+        return {"state": self.state, "state_slots": _h2d([self.bm.state_slot(i) for i in sids], torch.int32, self.device)}
+
+    def _state_copies(self) -> None:
+        """Carry out the slot copies that forks queued (children start from their prompt's state)."""
+        if self.state is not None:
+            self.state.copy_slots(self.bm.take_state_copies())
+
+    def _fork_children(self, g: SequenceGroup) -> None:
+        """Fork a prefilled prompt into the group's sequences and free the transient parent; the last child takes
+        over the parent's state slot, so a group never holds more slots than it has sequences."""
+        parent = -g.id
+        for i, s in enumerate(g.seqs):
+            self.bm.fork(parent, s.id, self.state is not None and i + 1 == len(g.seqs))
+        self._state_copies()
+        self.bm.free_sequence(parent)
 
     # ------------------------------------------------------------------ scheduling
     def _group_reservation(self, g: SequenceGroup) -> int:
@@ -599,14 +635,21 @@ class LLMEngine:
         g = self.waiting[0]
         live = sum(1 for s in self.running if not s.finished) + sum(x.n for x in self.prefilling)
         idle = not self.running and self.inflight is None and not self.prefilling
+        if self.state is not None and self._state_need(g) > self.bm.num_free_state_slots:
+            return False
         return live + g.n <= self.max_batch and ((self._group_reservation(g) <= self.free_blocks_unreserved
                                                   and self._physical_need(g) <= self.bm.num_free) or idle)
+
+    def _state_need(self, g: SequenceGroup) -> int:
+        return g.n
 
     def _admit(self) -> List[SequenceGroup]:
         out, tokens = [], 0
         while self.waiting:
             g = self.waiting[0]
             need = self._group_reservation(g)
+            if self.state is not None and sum(x.n for x in out) + g.n > self.bm.num_free_state_slots:
+                break
             if len(self.running) + sum(x.n for x in self.prefilling) + sum(x.n for x in out) + g.n > self.max_batch:
                 break
             phys = self._physical_need(g) + sum(self._physical_need(x) - self.kv_watermark for x in out)
@@ -678,7 +721,8 @@ class LLMEngine:
             # whole prompts (or their uncached tails) as portions over the paged cache, the mixed step's route
             k_lens = [len(p) for p in prompts]
             chunk_in = self._portion_tables([self.bm.block_table(pid) for pid in parents], cu, k_lens)
-            logits = self.model.forward_mixed(t_tok, t_pos, t_slots, self.cache, 0, None, chunk_in, t_last)
+            logits = self.model.forward_mixed(t_tok, t_pos, t_slots, self.cache, 0, None, chunk_in, t_last,
+                                              **self._state_args(parents))
         else:
             logits = self.model.prefill(t_tok, t_pos, t_slots, t_cu, max_len, t_last, self.cache, ctx=ctx)
         if use_cache:
@@ -697,6 +741,8 @@ class LLMEngine:
         (:meth:`add_request` with ``prefilled=``).  Must be called between steps."""
         if self.inflight is not None:
             raise RuntimeError("export_prefill while a decode step is in flight")
+        if self.state is not None:
+            raise RuntimeError("export_prefill: a prompt's recurrent state is not exported")
         parents = [-(1 << 40) - i for i in range(len(prompts))]
         need = sum((len(p) + self.block_size - 1) // self.block_size for p in prompts)
         if need > self.free_blocks_unreserved:
@@ -741,13 +787,11 @@ class LLMEngine:
         tokens from the prompt's last-token logits and add them to the running batch."""
         rows, seqs = [], []
         for g in groups:
-            parent = -g.id
+            self._fork_children(g)
             for s in g.seqs:
-                self.bm.fork(parent, s.id)
                 self._attach_rows(s)
                 rows.append(logits_of[g.id])
                 seqs.append(s)
-            self.bm.free_sequence(parent)
         if self.async_first_tokens and self.inflight is None and self.device.type == "cuda":
             self.inflight = self._launch_first(torch.stack(rows), seqs, groups)
             self.running.extend(seqs)
@@ -860,7 +904,8 @@ class LLMEngine:
             t_tok.index_copy_(0, from_prev[0], prev.tok_dev.index_select(0, from_prev[1]).to(torch.int32))
         logits = self.model.forward_mixed(t_tok, _h2d(pos, torch.int32, dev),
                                           _h2d(np.concatenate(slot_parts), torch.int32, dev), self.cache, B, dec_in,
-                                          chunk_in, _h2d(rows, torch.int64, dev))
+                                          chunk_in, _h2d(rows, torch.int64, dev),
+                                          **self._state_args([s.id for s in dec] + [-g.id for g, _, _ in items]))
         if prev is not None:  # host bookkeeping of the previous step while this forward runs
             with span("decode.process"):
                 events += self._process(prev)
@@ -883,12 +928,11 @@ class LLMEngine:
             ids = {g.id for g, _ in done}
             self.prefilling = [g for g in self.prefilling if g.id not in ids]
             for g, row in done:
+                self._fork_children(g)
                 for s in g.seqs:
-                    self.bm.fork(-g.id, s.id)
                     self._attach_rows(s)
                     children.append(s)
                     pick.append(row)
-                self.bm.free_sequence(-g.id)
         seqs = dec + children
         if seqs:
             sel = logits if pick == list(range(logits.shape[0])) else logits.index_select(
@@ -1138,23 +1182,31 @@ class LLMEngine:
         d = bk.d
         cascade = bool(bk.max_tiles) if cascade is None else cascade
 
+        extra = {} if self.state is None else {"state": self.state, "state_slots": d["state_slots"]}
+
         def fwd():
             return self.model.decode(d["tokens"], d["positions"], d["slots"], d["block_tables"], d["ctx_lens"],
                                      self.cache, num_splits=bk.splits,
-                                     cascade_tiles=d["tiles"] if cascade else None)
+                                     cascade_tiles=d["tiles"] if cascade else None, **extra)
 
         if not self.use_graphs:
             bk.logits = fwd()
             return
         g = bk.graphs.get(cascade)
-        if g is None and not bk.graphs and bk.B not in self.step_ab:
+        # (a recurrent model's step is not repeatable on the same inputs: no in-step A/B of plans for it)
+        if g is None and not bk.graphs and bk.B not in self.step_ab and self.state is None:
             self._step_ab(bk, fwd)
         if g is None:
             dev = self.device
             s = torch.cuda.Stream(device=dev)
             s.wait_stream(torch.cuda.current_stream(dev))
             with torch.cuda.stream(s):
+                if self.state is not None:  # the warm-up run advances the scratch slot, not the sequences' states
+                    real = d["state_slots"].clone()
+                    d["state_slots"].fill_(self.state.scratch)
                 fwd()  # warm-up (hipBLASLt heuristics, allocator) outside capture
+                if self.state is not None:
+                    d["state_slots"].copy_(real)
             torch.cuda.current_stream(dev).wait_stream(s)
             g = torch.cuda.CUDAGraph()
             # thread_local: another thread's device work during this capture (the K10b tally batcher's
@@ -1296,6 +1348,9 @@ class LLMEngine:
         prepare_decode_into(self.bm, [s.id for s in seqs], bk.width, bk.B, h["block_tables"], h["ctx_lens"],
                             h["slots"], h["positions"])
         st = self._static_inputs(seqs, key, bk)
+        if self.state is not None:
+            h["state_slots"][:] = self.state.scratch
+            h["state_slots"][:B] = [self.bm.state_slot(s.id) for s in seqs]
         if bk.host_static_key[parity] != key:
             for name in ("tiles", "seeds") + _F32_PARAMS + _I32_PARAMS:
                 h[name][...] = st[name]
@@ -1478,6 +1533,7 @@ class LLMEngine:
 
     def _swap_out(self, g: SequenceGroup) -> None:
         live = [s for s in g.seqs if not s.finished and self.bm.has_sequence(s.id)]
+        saved = self.state.take([self.bm.state_slot(s.id) for s in live]).cpu() if self.state is not None and live else None
         blocks, tables, lens = self.bm.swap_out([s.id for s in live])
         dev = self.device
         if blocks:
@@ -1490,7 +1546,7 @@ class LLMEngine:
         if dev.type == "cuda":
             ev = torch.cuda.Event()
             ev.record()
-        self.swapped.append(_SwapRecord(g, live, host, [list(t) for t in tables], list(lens), ev))
+        self.swapped.append(_SwapRecord(g, live, host, [list(t) for t in tables], list(lens), ev, saved))
         ids = {s.id for s in live}
         self.running = [s for s in self.running if s.id not in ids]
         self.free_blocks_unreserved += g.reserved_blocks
@@ -1509,12 +1565,16 @@ class LLMEngine:
             if (n + len(rec.seqs) + self.kv_watermark > self.bm.num_free
                     or (need > self.free_blocks_unreserved and (self.running or self.inflight is not None))):
                 return
+            if self.state is not None and len(rec.seqs) > self.bm.num_free_state_slots:
+                return
             self.swapped.popleft()
             phys = self.bm.swap_in([s.id for s in rec.seqs], n, rec.tables, rec.lens)
             if n:
                 dev = self.device
                 kv = rec.host.to(dev, non_blocking=True)
                 self.cache.put_blocks(torch.tensor(phys, dtype=torch.int64, device=dev), kv)
+            if self.state is not None and rec.state is not None:
+                self.state.put([self.bm.state_slot(s.id) for s in rec.seqs], rec.state)
             rec.group.reserved_blocks = need
             self.free_blocks_unreserved -= need
             self.running.extend(s for s in rec.seqs if not s.finished)

@@ -209,8 +209,158 @@ class MadipelConfig:
         return n
 
 
+
+# ------------------------------------------------------------------ Merudra
+@dataclass(frozen=True)
+class GatedAttentionSpec:
+    """Causal softmax attention without rotation: per-head unit-RMS q and k, the keys as projected are the values,
+    a query temperature that grows with the logarithm of the position, a sigmoid output gate."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    temp_coef: float
+    temp_every: int
+
+    @property
+    def nq(self) -> int:
+        return self.heads * self.dim
+
+    @property
+    def nk(self) -> int:
+        return self.kv_heads * self.dim
+
+    @property
+    def nv(self) -> int:
+        return self.kv_heads * self.vdim
+
+
+@dataclass(frozen=True)
+class DeltaRuleSpec:
+    """Gated delta rule: q, k over ``kv_heads`` heads of size ``dim``, v over ``heads`` heads of size ``vdim``,
+    each behind a short causal convolution with ``conv`` taps."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+
+    @property
+    def nq(self) -> int:
+        return self.kv_heads * self.dim
+
+    @property
+    def nv(self) -> int:
+        return self.heads * self.vdim
+
+
+@dataclass(frozen=True)
+class RoutedExpertsSpec:
+    experts: int       # real experts (each a gated feed-forward of inner width ff)
+    identity: int      # further router outputs whose expert is the identity
+    top: int
+    ff: int
+
+
+@dataclass(frozen=True)
+class MerudraLayerSpec:
+    type: str                                   # "attention" | "delta"
+    mixer: object                               # GatedAttentionSpec | DeltaRuleSpec
+    mlp: Optional[RoutedExpertsSpec]            # None: no feed-forward in this layer
+
+
+@dataclass(frozen=True)
+class MerudraConfig:
+    """Merudra: an fp32 residual stream; every sublayer reads x + causal_conv(x), its result is gated by
+    sigmoid(W x + b), RMS-normalised and added; mixers are gated causal attention or gated delta rule layers;
+    feed-forwards are routed experts with identity experts; a per-layer token embedding is added after the
+    feed-forward; the next layer reads a learned average of all earlier layers' results."""
+    name: str
+    vocab_size: int
+    hidden: int
+    layer_specs: Tuple[MerudraLayerSpec, ...]
+    norm_eps: float
+    canon_taps: int
+    side_dim: int
+    bos_token_id: int = 1
+    eos_token_id: int = 2
+
+    architecture = "Merudra"
+    num_experts = 0   # the engine's expert-parallel planning does not apply
+
+    @property
+    def layers(self) -> int:
+        return len(self.layer_specs)
+
+    @property
+    def attention_layers(self) -> Tuple[int, ...]:
+        return tuple(i for i, L in enumerate(self.layer_specs) if L.type == "attention")
+
+    @property
+    def heads(self) -> int:
+        return max(L.mixer.heads for L in self.layer_specs)
+
+    @property
+    def kv_heads(self) -> int:
+        return max(L.mixer.kv_heads for L in self.layer_specs)
+
+    @property
+    def head_dim(self) -> int:
+        return max(L.mixer.dim for L in self.layer_specs)
+
+    @classmethod
+    def from_dict(cls, c: dict, name: str = "merudra") -> "MerudraConfig":
+        specs = []
+        for L in c["layers"]:
+            m = L["mixer"]
+            if L["type"] == "attention":
+                t = m.get("q_temp") or {}
+                mixer = GatedAttentionSpec(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]),
+                                           vdim=int(m["vdim"]), scale=float(m["scale"]),
+                                           temp_coef=float(t.get("coef", 0.0)), temp_every=int(t.get("every", 0)))
+                if mixer.vdim != mixer.dim:
+                    raise ValueError("Merudra: the values are the keys, so vdim must equal dim")
+            elif L["type"] == "delta":
+                mixer = DeltaRuleSpec(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]),
+                                      vdim=int(m["vdim"]), conv=int(m["conv"]))
+            else:
+                raise ValueError(f"Merudra: unknown mixer type {L['type']!r}")
+            if mixer.heads % mixer.kv_heads:
+                raise ValueError("Merudra: heads must be a multiple of kv_heads")
+            mlp = L.get("mlp")
+            spec = None
+            if mlp is not None:
+                if mlp.get("kind") != "moe":
+                    raise ValueError(f"Merudra: unknown feed-forward kind {mlp.get('kind')!r}")
+                r = mlp["router"]
+                spec = RoutedExpertsSpec(experts=int(r["experts"]), identity=int(r.get("identity", 0)), top=int(r["top"]),
+                                         ff=int(mlp["expert"]["ff"]))
+                if not 1 <= spec.top <= spec.experts + spec.identity:
+                    raise ValueError("Merudra: router.top out of range")
+            specs.append(MerudraLayerSpec(L["type"], mixer, spec))
+        return cls(name=name, vocab_size=int(c["vocab"]), hidden=int(c["width"]), layer_specs=tuple(specs),
+                   norm_eps=float(c["norm"]["eps"]), canon_taps=int(c["canon"]["taps"]),
+                   side_dim=int(c["token_side"]["dim"]))
+
+    def params(self) -> int:
+        d = self.hidden
+        n = 2 * self.vocab_size * d + d + self.vocab_size * self.side_dim * self.layers
+        for i, L in enumerate(self.layer_specs):
+            m = L.mixer
+            n += 2 * d + 2 * d * self.canon_taps + 2 * (d * d + d) + (i + 2) + 2 * d * self.side_dim + d
+            if L.type == "attention":
+                n += d * (2 * m.nq + m.nk) + m.nq + m.nk + d * m.heads * m.vdim
+            else:
+                n += d * (2 * m.nq + 2 * m.nv + 2 * m.heads) + (2 * m.nq + m.nv) * m.conv + 2 * m.heads + m.vdim + d * m.nv
+            if L.mlp is not None:
+                e = L.mlp
+                n += e.experts * 3 * d * e.ff + (e.experts + e.identity) * (d + 1)
+        return n
+
+
 # config.json "architecture" -> config class of the layer-list decoders
-ARCHITECTURES = {"Madipel": MadipelConfig}
+ARCHITECTURES = {"Madipel": MadipelConfig, "Merudra": MerudraConfig}
 
 
 def load_model_config(model_dir) -> object:

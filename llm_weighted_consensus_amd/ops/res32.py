@@ -128,3 +128,130 @@ def window_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, p
 
 def softplus(x: float) -> float:
     return max(x, 0.0) + math.log1p(math.exp(-abs(x)))
+
+
+# ------------------------------------------------------------------ recurrent state, gated layers, routed experts
+class StepItems:
+    """A step's rows grouped by sequence for the kernels that carry per-sequence state: item i owns rows
+    [cu[i], cu[i+1]) at consecutive positions and the state slot ``slots[i]`` (a decode row is an item of one
+    row).  All int32 device tensors; ``row_item[t]`` is the item of row t."""
+
+    def __init__(self, row_item: torch.Tensor, cu: torch.Tensor, slots: torch.Tensor, positions: torch.Tensor):
+        self.row_item, self.cu, self.slots, self.positions = row_item, cu, slots, positions
+
+    @classmethod
+    def rows(cls, slots: torch.Tensor, positions: torch.Tensor) -> "StepItems":
+        """Every row its own item (a decode step); built from device tensors only (capturable)."""
+        n = positions.numel()
+        ar = torch.arange(n + 1, dtype=torch.int32, device=positions.device)
+        return cls(ar[:n], ar, slots, positions)
+
+
+def conv_hist(x: torch.Tensor, w: torch.Tensor, hist: torch.Tensor, items: StepItems, out: torch.Tensor,
+              mode: int = 0, out2: Optional[torch.Tensor] = None, update: bool = True) -> torch.Tensor:
+    """Causal convolution over time per channel with the inputs before a portion's first row taken from the
+    sequence's slot of ``hist`` (fp32 [slots, taps - 1, C]); ``w`` fp32 [C, taps], last column = the current
+    row's.  ``mode`` 0: out = x + conv(x) (``out2``: a copy of x in out's dtype); 1: out = silu(conv(x)).
+    With ``update`` the slot then holds the last taps - 1 inputs after this step."""
+    K = kernels()
+    K.conv_hist(x, w, hist, items.row_item, items.cu, items.slots, items.positions, out, out2, int(mode))
+    if update:
+        K.conv_hist_update(x, hist, items.cu, items.slots, int(w.shape[1]))
+    return out
+
+
+def delta_rule(qkv: torch.Tensor, ba: torch.Tensor, b_off: int, a_off: int, A_log: torch.Tensor, dt_bias: torch.Tensor,
+               state: torch.Tensor, items: StepItems, H: int, G: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Gated delta rule over a step's items: per head S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q
+    with q, k unit vectors per head (q times D^-1/2), beta = sigmoid(ba[:, b_off + h]),
+    g = exp(-exp(A_log_h) softplus(ba[:, a_off + h] + dt_bias_h)).  ``qkv`` fp32 [T, 2 G D + H Dv] (after the
+    short convolutions), ``state`` fp32 [slots, H, D, Dv] (read unless the item starts at position 0, written
+    back).  Returns o fp32 [T, H Dv]."""
+    if out is None:
+        out = torch.empty(qkv.shape[0], H * state.shape[3], dtype=torch.float32, device=qkv.device)
+    kernels().delta_rule(qkv, ba, int(b_off), int(a_off), A_log, dt_bias, state, items.cu, items.slots, items.positions,
+                         out, int(H), int(G))
+    return out
+
+
+def head_norm_gate(o: torch.Tensor, out: torch.Tensor, H: int, eps: float, w: Optional[torch.Tensor] = None,
+                   gate: Optional[torch.Tensor] = None, mode: str = "silu") -> torch.Tensor:
+    """out = o / rms(o) per head * w * act(gate); o fp32 [T, H Dv], ``mode`` silu | sigmoid (ignored without gate)."""
+    kernels().head_norm_gate(o, gate, w, out, int(H), float(eps), 0 if gate is None else (1 if mode == "silu" else 2))
+    return out
+
+
+def embed_rows(table: torch.Tensor, tokens: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x[t] = table[tokens[t]] as fp32."""
+    if out is None:
+        out = torch.empty(tokens.numel(), table.shape[1], dtype=torch.float32, device=table.device)
+    kernels().embed_rows(table, tokens, out)
+    return out
+
+
+def head_norm_kv_write(proj: torch.Tensor, k_off: int, v_off: int, positions: torch.Tensor, slots: torch.Tensor,
+                       k_cache: torch.Tensor, v_cache: torch.Tensor, H: int, G: int, eps: float, scale: float,
+                       temp_coef: float = 0.0, temp_every: int = 0, q_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """From fused projection rows (q at column 0, k at ``k_off``, values at ``v_off``; ``v_off == k_off``: the
+    keys as projected are the values): q and k divided by their root mean square per head; q times
+    ``scale * (1 + temp_coef ln(floor((p + 1) / temp_every) + 1))`` into an fp32 buffer (returned); the normalised k
+    and the values into the paged cache at ``slots`` (-1: no write)."""
+    D = k_cache.shape[2] // G
+    if q_out is None:
+        q_out = torch.empty(proj.shape[0], H * D, dtype=torch.float32, device=proj.device)
+    kernels().head_norm_kv_write(proj, int(k_off), int(v_off), positions, slots, q_out, k_cache, v_cache, int(H), int(G),
+                                 float(eps), float(scale), float(temp_coef), int(temp_every))
+    return q_out
+
+
+def gate_mul(a: torch.Tensor, g: torch.Tensor, mode: str = "sigmoid") -> torch.Tensor:
+    """a *= sigmoid(g) (or silu(g)) in place; both may be column slices of row-dense buffers."""
+    kernels().gate_mul(a, g, 0 if mode == "sigmoid" else 1)
+    return a
+
+
+def gated_norm_residual(x: torch.Tensor, y: torch.Tensor, w: torch.Tensor, eps: float,
+                        gate_logits: Optional[torch.Tensor] = None, x_cast: Optional[torch.Tensor] = None) -> None:
+    """x (fp32) += z / rms(z) * w with z = y * sigmoid(gate_logits) (z = y without); w fp32.  ``x_cast`` (bf16
+    [T, d]) also receives the new x."""
+    kernels().gated_norm_residual(x, y, gate_logits, w, x_cast, float(eps))
+
+
+def rmsnorm_rows(x: torch.Tensor, w: torch.Tensor, eps: float, dtype, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """RMS norm of fp32 rows (optionally the gathered ``rows``, int64) with fp32 weight -> ``dtype`` rows."""
+    n = x.shape[0] if rows is None else rows.numel()
+    out = torch.empty(n, x.shape[1], dtype=dtype, device=x.device)
+    kernels().rmsnorm_rows(x, rows, w, out, float(eps))
+    return out
+
+
+def gelu_mul_rows(z: torch.Tensor, table: torch.Tensor, off: int, tokens: torch.Tensor) -> torch.Tensor:
+    """gelu_tanh(z[t]) * table[tokens[t], off : off + n] for z [T, n]."""
+    out = torch.empty(z.shape[0], z.shape[1], dtype=z.dtype, device=z.device)
+    kernels().gelu_mul_rows(z, table, int(off), tokens, out)
+    return out
+
+
+def stack_mix(X: torch.Tensor, coef: torch.Tensor, n: int, out: torch.Tensor) -> torch.Tensor:
+    """out = sum_{j < n} coef[j] X[j] over a stack of fp32 streams X [>= n, T, d]."""
+    kernels().stack_mix(X, coef, int(n), out)
+    return out
+
+
+def router(z: torch.Tensor, correction: torch.Tensor, experts: int, top: int):
+    """Softmax router over all outputs of ``z`` (fp32 [T, NE]); the ``top`` largest of softmax + correction are
+    chosen, weighted by their softmax (not renormalised).  Outputs >= ``experts`` are identity experts.  Returns
+    (ids [T, top], w [T, top], row_off [experts + 1], src [T top], row_expert [T top], inv [T top]): expert-major
+    row r holds token src[r] for expert row_expert[r]; choice (t, j) is row inv[t top + j], -1 for an identity."""
+    return tuple(kernels().router(z, correction, int(experts), int(top)))
+
+
+def expert_rows(h: torch.Tensor, src: torch.Tensor, row_expert: torch.Tensor, row_off: torch.Tensor, w_gu: torch.Tensor,
+                w_down: torch.Tensor) -> torch.Tensor:
+    """Y[r] = W_down[e] (silu(W_gate[e] h) * (W_up[e] h)) for every expert-major row r (fp32 sums, any sizes)."""
+    return kernels().expert_rows(h, src, row_expert, row_off, w_gu, w_down)
+
+
+def moe_combine(Y: torch.Tensor, inv: torch.Tensor, w: torch.Tensor, h: torch.Tensor) -> torch.Tensor:
+    """fp32 [T, d]: sum_j w[t, j] * (Y[inv[t, j]] if inv >= 0 else h[t])."""
+    return kernels().moe_combine(Y, inv, w, h)
