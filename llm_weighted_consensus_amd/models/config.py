@@ -348,13 +348,14 @@ class MerudraConfig:
         n = 2 * self.vocab_size * d + d + self.vocab_size * self.side_dim * self.layers
         for i, L in enumerate(self.layer_specs):
             m = L.mixer
-            n += 2 * d + 2 * d * self.canon_taps + 2 * (d * d + d) + (i + 2) + 2 * d * self.side_dim + d
+            n += d + d * self.canon_taps + (d * d + d) + (i + 2) + 2 * d * self.side_dim + d
             if L.type == "attention":
                 n += d * (2 * m.nq + m.nk) + m.nq + m.nk + d * m.heads * m.vdim
             else:
                 n += d * (2 * m.nq + 2 * m.nv + 2 * m.heads) + (2 * m.nq + m.nv) * m.conv + 2 * m.heads + m.vdim + d * m.nv
             if L.mlp is not None:
                 e = L.mlp
+                n += d + d * self.canon_taps + (d * d + d)
                 n += e.experts * 3 * d * e.ff + (e.experts + e.identity) * (d + 1)
         return n
 

@@ -155,3 +155,59 @@ def forward(cfg, W, tokens, layers_out=None):
         if layers_out is not None:
             layers_out.append(x)
     return (rms_unit(x, eps) * W["final.norm"]) @ W["head"].T
+
+
+# ------------------------------------------------------------------ test models
+def make_config(width, vocab, layers, taps=3, side=5, eps=1e-5):
+    """config.json of a small model.  ``layers``: dicts with type, heads, kv_heads, dim, vdim and, for attention,
+    scale / coef / every; for delta, conv; ``mlp``: None or dict(experts, identity, top, ff)."""
+    out = []
+    for L in layers:
+        if L["type"] == "attention":
+            mixer = {"heads": L["heads"], "kv_heads": L["kv_heads"], "dim": L["dim"], "vdim": L["dim"], "scale": L.get("scale", 0.3),
+                     "q_temp": {"coef": L.get("coef", 0.4), "every": L.get("every", 7)}}
+        else:
+            mixer = {"heads": L["heads"], "kv_heads": L["kv_heads"], "dim": L["dim"], "vdim": L["vdim"], "conv": L.get("conv", 4)}
+        m = L.get("mlp")
+        mlp = None if m is None else {"kind": "moe", "expert": {"ff": m["ff"]},
+                                      "router": {"experts": m["experts"], "identity": m["identity"], "top": m["top"]}}
+        out.append({"type": L["type"], "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Merudra", "canon": {"taps": taps}, "layers": out, "norm": {"eps": eps},
+            "token_side": {"dim": side}, "vocab": vocab, "width": width}
+
+
+def make_weights(cfg, seed):
+    """Random bf16 tensors under the checkpoint's names; scales chosen so that every mechanism matters."""
+    g = torch.Generator().manual_seed(seed)
+    d, V, taps, sd = cfg["width"], cfg["vocab"], cfg["canon"]["taps"], cfg["token_side"]["dim"]
+
+    def rn(*shape, s=1.0):
+        return torch.randn(*shape, generator=g) * s
+
+    def lin(o, i):
+        return rn(o, i, s=i ** -0.5)
+
+    W = {"embed": rn(V, d), "side.embed": rn(V, sd * len(cfg["layers"])), "final.norm": 1 + rn(d, s=0.1), "head": lin(V, d)}
+    for i, L in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", L["mixer"]
+        H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        W.update({p + "norm1": 1 + rn(d, s=0.1), p + "canon1": rn(d, taps, s=0.3), p + "rg1": lin(d, d), p + "rg1.b": rn(d, s=0.3),
+                  p + "dwa": rn(i + 2, s=0.3), p + "side.gate": lin(sd, d), p + "side.proj": lin(d, sd), p + "side.norm": 1 + rn(d, s=0.1)})
+        W[p + "dwa"][-1] += 1.0
+        if L["type"] == "attention":
+            W.update({p + "mix.q": lin(H * D, d), p + "mix.q.b": rn(H * D, s=0.2), p + "mix.k": lin(G * D, d),
+                      p + "mix.k.b": rn(G * D, s=0.2), p + "mix.g": lin(H * Dv, d), p + "mix.o": lin(d, H * Dv)})
+        else:
+            c = m["conv"]
+            W.update({p + "mix.q": lin(G * D, d), p + "mix.q.conv": rn(G * D, c, s=0.6), p + "mix.k": lin(G * D, d),
+                      p + "mix.k.conv": rn(G * D, c, s=0.6), p + "mix.v": lin(H * Dv, d), p + "mix.v.conv": rn(H * Dv, c, s=0.6),
+                      p + "mix.b": lin(H, d), p + "mix.a": lin(H, d), p + "mix.A_log": rn(H, s=0.7), p + "mix.dt_bias": rn(H),
+                      p + "mix.norm": 1 + rn(Dv, s=0.1), p + "mix.g": lin(H * Dv, d), p + "mix.o": lin(d, H * Dv)})
+        if L["mlp"] is not None:
+            r, ff = L["mlp"]["router"], L["mlp"]["expert"]["ff"]
+            ne = r["experts"] + r["identity"]
+            W.update({p + "norm2": 1 + rn(d, s=0.1), p + "canon2": rn(d, taps, s=0.3), p + "rg2": lin(d, d), p + "rg2.b": rn(d, s=0.3),
+                      p + "mlp.router": lin(ne, d) * 2, p + "mlp.correction": rn(ne, s=0.15)})
+            for e in range(r["experts"]):
+                W.update({f"{p}mlp.e{e}.gate": lin(ff, d), f"{p}mlp.e{e}.up": lin(ff, d), f"{p}mlp.e{e}.down": lin(d, ff)})
+    return {k: v.to(torch.bfloat16) for k, v in W.items()}
