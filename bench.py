@@ -56,7 +56,9 @@ def parse():
     ap.add_argument("--sizes", default="small,8b-layer", help="--compare-decoders: sizes to run")
     ap.add_argument("--compare-layers", type=int, default=4, help="--compare-decoders: layers per model")
     ap.add_argument("--window", type=int, default=0, help="--compare-decoders: Madipel's window (0: the whole context)")
-    ap.add_argument("--designs", default="madipel,llama", help="--compare-decoders: designs to run")
+    ap.add_argument("--designs", default="madipel,llama",
+                    help="--compare-decoders: designs to run (madipel, llama, merudra, mixtral)")
+    ap.add_argument("--pattern", default="ad", help="--compare-decoders: Merudra's layer kinds, a(ttention) / d(elta), repeated")
     return ap.parse_args()
 
 
@@ -66,7 +68,7 @@ def main():
     if a.compare_decoders:
         import bench_decoders
 
-        sys.exit(bench_decoders.run(a.sizes, a.compare_layers, prompt_len=2048, window=a.window, designs=a.designs))
+        sys.exit(bench_decoders.run(a.sizes, a.compare_layers, prompt_len=2048, window=a.window, designs=a.designs, pattern=a.pattern))
     from llm_weighted_consensus_amd.parallel import launch
 
     # `python bench.py --gpus N` without torchrun: this process only launches N ranks (never touches the GPU)

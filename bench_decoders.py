@@ -3,6 +3,10 @@
 
     python bench.py --compare-decoders [--sizes small,8b-layer] [--compare-layers 4]
 
+Designs: ``madipel``, ``llama``, ``merudra``, ``mixtral`` (``--designs merudra,mixtral`` puts Merudra beside the
+closest existing decoder, the routed-experts Mixtral: 8 experts, 2 per token, the same active feed-forward width;
+Merudra's layers alternate attention and gated delta rule mixers and add 2 identity experts).
+
 For each size a Madipel model (parallel layers, windowed attention with distance bias, xIELU feed-forward, fp32
 residual) and the closest existing decoder (Llama: sequential layers, causal GQA attention with RoPE, SwiGLU) are
 built with random weights at the same width, layer count, head counts, head size, vocabulary and parameter count
@@ -46,6 +50,33 @@ def _llama(size: dict, layers: int, max_pos: int, device, seed: int):
     return LlamaModel(cfg, device=device, seed=seed, max_position=max_pos)
 
 
+def _merudra(size: dict, layers: int, device, seed: int, experts: int = 8, top: int = 2, pattern: str = "ad"):
+    """Attention and delta layers alternating (``pattern``: a / d per layer, repeated), routed experts of inner width
+    ffn / top (the active feed-forward width of the dense models), two identity experts."""
+    from llm_weighted_consensus_amd.models.config import MerudraConfig
+    from llm_weighted_consensus_amd.models.merudra import MerudraModel
+
+    H, G, D = size["heads"], size["kv_heads"], size["head_dim"]
+    mlp = {"kind": "moe", "expert": {"ff": size["ffn"] // top}, "router": {"experts": experts, "identity": 2, "top": top}}
+    att = {"type": "attention", "mlp": mlp,
+           "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "q_temp": {"coef": 0.1, "every": 512}}}
+    dlt = {"type": "delta", "mlp": mlp, "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "conv": 4}}
+    cfg = MerudraConfig.from_dict({"architecture": "Merudra", "canon": {"taps": 4},
+                                   "layers": [att if pattern[i % len(pattern)] == "a" else dlt for i in range(layers)],
+                                   "norm": {"eps": 1e-5}, "token_side": {"dim": 64}, "vocab": size["vocab"],
+                                   "width": size["width"]}, name="merudra-bench")
+    return MerudraModel(cfg, device=device, seed=seed)
+
+
+def _mixtral(size: dict, layers: int, max_pos: int, device, seed: int, experts: int = 8, top: int = 2):
+    from llm_weighted_consensus_amd.models.config import DecoderConfig
+    from llm_weighted_consensus_amd.models.mixtral import MixtralModel
+
+    cfg = DecoderConfig("mixtral-bench", size["vocab"], size["width"], layers, size["heads"], size["kv_heads"],
+                        size["head_dim"], size["ffn"] // top, max_position=max_pos, num_experts=experts, experts_per_token=top)
+    return MixtralModel(cfg, device=device, seed=seed, max_position=max_pos)
+
+
 def _measure(model, prompt_len: int, n_prompts: int, batch: int, gen: int, reps: int) -> dict:
     import torch
 
@@ -83,7 +114,7 @@ def _measure(model, prompt_len: int, n_prompts: int, batch: int, gen: int, reps:
 
 
 def run(sizes: str = "small,8b-layer", layers: int = 4, prompt_len: int = 2048, n_prompts: int = 8, batch: int = 64,
-        gen: int = 33, window: int = 0, reps: int = 2, designs: str = "madipel,llama") -> int:
+        gen: int = 33, window: int = 0, reps: int = 2, designs: str = "madipel,llama", pattern: str = "ad") -> int:
     import torch
 
     dev = torch.device("cuda", 0)
@@ -93,8 +124,14 @@ def run(sizes: str = "small,8b-layer", layers: int = 4, prompt_len: int = 2048, 
     for name in sizes.split(","):
         size = SIZES[name]
         for design in designs.split(","):
-            model = (_madipel(size, layers, window, dev, 3) if design == "madipel"
-                     else _llama(size, layers, prompt_len + gen + 80, dev, 3))
+            if design == "madipel":
+                model = _madipel(size, layers, window, dev, 3)
+            elif design == "merudra":
+                model = _merudra(size, layers, dev, 3, pattern=pattern)
+            elif design == "mixtral":
+                model = _mixtral(size, layers, prompt_len + gen + 80, dev, 3)
+            else:
+                model = _llama(size, layers, prompt_len + gen + 80, dev, 3)
             r = _measure(model, prompt_len, n_prompts, batch, gen, reps)
             params = model.cfg.params()
             del model
@@ -104,12 +141,14 @@ def run(sizes: str = "small,8b-layer", layers: int = 4, prompt_len: int = 2048, 
                     **{k: round(v, 3) for k, v in r.items()}, "dtype": "bf16", "data": "synthetic"}
             print(json.dumps(line), flush=True)
             summary.setdefault(name, {})[design] = r
-    out = {}
-    for name, d in summary.items():
-        if "madipel" in d and "llama" in d:
-            out[name] = {"prefill_ratio": round(d["madipel"]["prefill_tok_s"] / d["llama"]["prefill_tok_s"], 3),
-                         "decode_ratio": round(d["madipel"]["decode_tok_s"] / d["llama"]["decode_tok_s"], 3)}
-    print(json.dumps({"bench": "compare-decoders", "madipel_over_llama": out}), flush=True)
+    for a, b in (("madipel", "llama"), ("merudra", "mixtral"), ("merudra", "madipel")):
+        out = {}
+        for name, d in summary.items():
+            if a in d and b in d:
+                out[name] = {"prefill_ratio": round(d[a]["prefill_tok_s"] / d[b]["prefill_tok_s"], 3),
+                             "decode_ratio": round(d[a]["decode_tok_s"] / d[b]["decode_tok_s"], 3)}
+        if out:
+            print(json.dumps({"bench": "compare-decoders", f"{a}_over_{b}": out}), flush=True)
     return 0
 
 

@@ -28,8 +28,8 @@ int r32_conv_hist(const void*, int, const float*, const float*, long long, const
                   void*, int, void*, int, int, int, int, int, int, hipStream_t);
 int r32_conv_hist_update(const void*, int, float*, long long, const int*, const int*, int, int, int, int, hipStream_t);
 int r32_delta_rule_max_dim();
-int r32_delta_rule(const float*, int, const void*, int, int, int, const float*, const float*, float*, long long, const int*,
-                   const int*, const int*, float*, int, int, int, int, int, int, int, hipStream_t);
+int r32_delta_rule(float*, int, const void*, int, int, int, const float*, const float*, float*, float*, long long, const int*,
+                   const int*, const int*, float*, int, int, int, int, int, int, int, int, hipStream_t);
 int r32_head_norm_gate(const float*, int, const void*, int, const float*, void*, int, int, int, int, float, int, int,
                        hipStream_t);
 int r32_embed_rows(const void*, const int*, float*, int, int, int, int, hipStream_t);
@@ -223,13 +223,14 @@ bool window_attn_mfma_ok(int64_t D, int64_t Dv) { return r32_window_attn_mfma_ok
 // i - j), cu_q / k_lens int32 per item (k_lens: the sequence's length after this step), max_q the longest portion.
 // Positions ascend by one along each item's rows.
 void window_attn_mfma(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, Tensor cu_q, Tensor k_lens,
-                      int64_t max_q, Tensor block_tables, Tensor bias, int64_t window, Tensor out, int64_t H, int64_t G) {
+                      int64_t max_q, Tensor block_tables, c10::optional<Tensor> bias, int64_t window, Tensor out, int64_t H,
+                      int64_t G) {
   want(q, torch::kFloat32, "window_attn_mfma q");
   want(positions, torch::kInt32, "window_attn_mfma positions");
   want(block_tables, torch::kInt32, "window_attn_mfma block_tables");
   want(cu_q, torch::kInt32, "window_attn_mfma cu_q");
   want(k_lens, torch::kInt32, "window_attn_mfma k_lens");
-  want(bias, torch::kFloat32, "window_attn_mfma bias");
+  if (bias.has_value()) want(*bias, torch::kFloat32, "window_attn_mfma bias");
   TORCH_CHECK(k_cache.is_cuda() && v_cache.is_cuda() && out.is_cuda() && k_cache.scalar_type() == torch::kBFloat16 &&
                   v_cache.scalar_type() == torch::kBFloat16 && out.scalar_type() == torch::kBFloat16,
               "window_attn_mfma: bf16 caches and out");
@@ -245,22 +246,22 @@ void window_attn_mfma(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions
   const int items = (int)block_tables.size(0);
   TORCH_CHECK(block_tables.dim() == 2 && cu_q.numel() == items + 1 && k_lens.numel() == items && max_q >= 1 &&
                   q.numel() == (int64_t)T * H * D && out.size(0) == T && out.size(1) == H * Dv && window >= 1 &&
-                  bias.numel() == H * window, "window_attn_mfma: shapes disagree");
+                  (!bias.has_value() || bias->numel() == H * window), "window_attn_mfma: shapes disagree");
   done(r32_window_attn_mfma(q.data_ptr<float>(), k_cache.data_ptr(), v_cache.data_ptr(), (long long)k_cache.stride(0),
                             (long long)v_cache.stride(0), BS, positions.data_ptr<int>(), cu_q.data_ptr<int>(),
                             k_lens.data_ptr<int>(), items, (int)max_q, block_tables.data_ptr<int>(),
-                            (int)block_tables.size(1), bias.data_ptr<float>(), (int)window, out.data_ptr(), ldo, (int)H, (int)G,
-                            D, Dv, stream()), "window_attn_mfma");
+                            (int)block_tables.size(1), bias.has_value() ? bias->data_ptr<float>() : nullptr, (int)window,
+                            out.data_ptr(), ldo, (int)H, (int)G, D, Dv, stream()), "window_attn_mfma");
 }
 
 // One new token per sequence on the matrix cores (bf16 caches): row b reads table row b, its key range ends at
 // positions[b].  max_keys: a host-side upper bound of the keys a row sees (min(window, longest context)).
-void window_attn_decode(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, Tensor block_tables, Tensor bias,
-                        int64_t window, int64_t max_keys, Tensor out, int64_t H, int64_t G) {
+void window_attn_decode(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, Tensor block_tables,
+                        c10::optional<Tensor> bias, int64_t window, int64_t max_keys, Tensor out, int64_t H, int64_t G) {
   want(q, torch::kFloat32, "window_attn_decode q");
   want(positions, torch::kInt32, "window_attn_decode positions");
   want(block_tables, torch::kInt32, "window_attn_decode block_tables");
-  want(bias, torch::kFloat32, "window_attn_decode bias");
+  if (bias.has_value()) want(*bias, torch::kFloat32, "window_attn_decode bias");
   TORCH_CHECK(k_cache.is_cuda() && v_cache.is_cuda() && out.is_cuda() && k_cache.scalar_type() == torch::kBFloat16 &&
                   v_cache.scalar_type() == torch::kBFloat16 && out.scalar_type() == torch::kBFloat16,
               "window_attn_decode: bf16 caches and out");
@@ -274,14 +275,15 @@ void window_attn_decode(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positio
   TORCH_CHECK(k_cache.stride(0) % 8 == 0 && v_cache.stride(0) % 8 == 0 && ((uintptr_t)k_cache.data_ptr() & 15) == 0 &&
                   ((uintptr_t)v_cache.data_ptr() & 15) == 0, "window_attn_decode: cache alignment");
   TORCH_CHECK(block_tables.dim() == 2 && block_tables.size(0) >= B && q.numel() == (int64_t)B * H * D && out.size(0) == B &&
-                  out.size(1) == H * Dv && window >= 1 && max_keys >= 1 && bias.numel() == H * window,
+                  out.size(1) == H * Dv && window >= 1 && max_keys >= 1 && (!bias.has_value() || bias->numel() == H * window),
               "window_attn_decode: shapes disagree");
   const int S = r32_window_attn_decode_splits(B, (int)G, (int)(H / G), (int)max_keys);
   auto part = torch::empty({(int64_t)B * H * S * (Dv + 2)}, q.options());
   float* po = part.data_ptr<float>();
   done(r32_window_attn_decode(q.data_ptr<float>(), k_cache.data_ptr(), v_cache.data_ptr(), (long long)k_cache.stride(0),
                               (long long)v_cache.stride(0), BS, positions.data_ptr<int>(), block_tables.data_ptr<int>(),
-                              (int)block_tables.size(1), bias.data_ptr<float>(), (int)window, po, po + (int64_t)B * H * S * Dv, S,
+                              (int)block_tables.size(1), bias.has_value() ? bias->data_ptr<float>() : nullptr, (int)window, po,
+                              po + (int64_t)B * H * S * Dv, S,
                               (int)max_keys, out.data_ptr(), ldo, B, (int)H, (int)G, D, Dv, stream()), "window_attn_decode");
 }
 
@@ -350,7 +352,7 @@ void conv_hist_update(Tensor x, Tensor hist, Tensor cu, Tensor item_slot, int64_
 
 int64_t delta_rule_max_dim() { return r32_delta_rule_max_dim(); }
 
-// qkv fp32 [T, 2 G D + H Dv]; ba [T, ...] with beta logits at b_off and decay inputs at a_off (H columns each);
+// qkv fp32 [T, 2 G D + H Dv] (its q and k columns are normalised in place); ba [T, ...] with beta logits at b_off and decay inputs at a_off (H columns each);
 // state fp32 [slots, H, D, Dv] view; out fp32 [T, H Dv]
 void delta_rule(Tensor qkv, Tensor ba, int64_t b_off, int64_t a_off, Tensor A_log, Tensor dt_bias, Tensor state, Tensor cu,
                 Tensor item_slot, Tensor positions, Tensor out, int64_t H, int64_t G) {
@@ -373,10 +375,11 @@ void delta_rule(Tensor qkv, Tensor ba, int64_t b_off, int64_t a_off, Tensor A_lo
                   ba.size(0) == T && b_off >= 0 && a_off >= 0 && b_off + H <= ba.size(1) && a_off + H <= ba.size(1) &&
                   A_log.numel() == H && dt_bias.numel() == H && positions.numel() == T && cu.numel() == item_slot.numel() + 1 &&
                   D <= r32_delta_rule_max_dim(), "delta_rule: shapes disagree");
+  Tensor bg = torch::empty({T, 2 * H}, qkv.options());
   done(r32_delta_rule(qkv.data_ptr<float>(), ldq, ba.data_ptr(), ldb, (int)b_off, (int)a_off, A_log.data_ptr<float>(),
-                      dt_bias.data_ptr<float>(), state.data_ptr<float>(), (long long)state.stride(0), cu.data_ptr<int>(),
-                      item_slot.data_ptr<int>(), positions.data_ptr<int>(), out.data_ptr<float>(), ldo, (int)item_slot.numel(),
-                      (int)H, (int)G, D, Dv, f, stream()), "delta_rule");
+                      dt_bias.data_ptr<float>(), bg.data_ptr<float>(), state.data_ptr<float>(), (long long)state.stride(0),
+                      cu.data_ptr<int>(), item_slot.data_ptr<int>(), positions.data_ptr<int>(), out.data_ptr<float>(), ldo, T,
+                      (int)item_slot.numel(), (int)H, (int)G, D, Dv, f, stream()), "delta_rule");
 }
 
 // o fp32 [T, H Dv]; gate (mode 1 silu, 2 sigmoid; 0: unused) and out of the activation dtype; w fp32 [Dv] or absent

@@ -15,6 +15,7 @@ namespace {
 
 constexpr int kMaxPerLane = 8;  // router outputs per lane: NE <= 512
 
+template <int PER>
 __global__ void router_topk_kernel(const float* __restrict__ z, const float* __restrict__ corr, int NE, int E, int k,
                                    int* __restrict__ ids, float* __restrict__ wts, int* __restrict__ counts,
                                    int* __restrict__ rank, int T) {
@@ -22,10 +23,10 @@ __global__ void router_topk_kernel(const float* __restrict__ z, const float* __r
   if (t >= T) return;
   const int lane = threadIdx.x & 63;
   const float* zr = z + (size_t)t * NE;
-  float v[kMaxPerLane], c[kMaxPerLane];
+  float v[PER], c[PER];
   float m = -INFINITY;
 #pragma unroll
-  for (int i = 0; i < kMaxPerLane; ++i) {
+  for (int i = 0; i < PER; ++i) {
     const int e = lane + 64 * i;
     v[i] = e < NE ? zr[e] : -INFINITY;
     m = fmaxf(m, v[i]);
@@ -33,14 +34,14 @@ __global__ void router_topk_kernel(const float* __restrict__ z, const float* __r
   m = wave_max(m);
   float sum = 0.f;
 #pragma unroll
-  for (int i = 0; i < kMaxPerLane; ++i) {
+  for (int i = 0; i < PER; ++i) {
     const int e = lane + 64 * i;
     v[i] = e < NE ? expf(v[i] - m) : 0.f;
     sum += v[i];
   }
   sum = wave_sum(sum);
 #pragma unroll
-  for (int i = 0; i < kMaxPerLane; ++i) {
+  for (int i = 0; i < PER; ++i) {
     const int e = lane + 64 * i;
     v[i] = v[i] / sum;
     c[i] = e < NE ? v[i] + corr[e] : -INFINITY;
@@ -49,7 +50,7 @@ __global__ void router_topk_kernel(const float* __restrict__ z, const float* __r
     float best = -INFINITY;
     int bi = 0x7fffffff;
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i) {
+    for (int i = 0; i < PER; ++i) {
       const int e = lane + 64 * i;
       if (e < NE && (c[i] > best || (c[i] == best && e < bi))) best = c[i], bi = e;
     }
@@ -62,7 +63,7 @@ __global__ void router_topk_kernel(const float* __restrict__ z, const float* __r
     // the winner's lane removes it and reports its score
     float sc = 0.f;
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i)
+    for (int i = 0; i < PER; ++i)
       if (lane + 64 * i == bi) sc = v[i], c[i] = -INFINITY;
     sc = wave_sum(sc);
     if (lane == 0) {
@@ -167,7 +168,8 @@ extern "C" int r32_router(const float* z, const float* corr, int T, int NE, int 
                           int* rank, int* row_off, int* src, int* row_expert, int* inv, hipStream_t s) {
   if (T <= 0) return 0;
   if (NE > 64 * kMaxPerLane || k < 1 || k > NE || E > NE) return -1;
-  router_topk_kernel<<<(T + 3) / 4, 256, 0, s>>>(z, corr, NE, E, k, ids, wts, counts, rank, T);
+  if (NE <= 64) router_topk_kernel<1><<<(T + 3) / 4, 256, 0, s>>>(z, corr, NE, E, k, ids, wts, counts, rank, T);
+  else router_topk_kernel<kMaxPerLane><<<(T + 3) / 4, 256, 0, s>>>(z, corr, NE, E, k, ids, wts, counts, rank, T);
   router_offsets_kernel<<<1, 64, 0, s>>>(counts, E, row_off);
   const int total = T * k;
   router_scatter_kernel<<<(total + 255) / 256, 256, 0, s>>>(ids, rank, row_off, E, k, src, row_expert, inv, total);

@@ -8,7 +8,7 @@
 //                     inputs before the item's first row come from the slot's history (the last taps-1 inputs).
 //                     MODE 0: out = x + y (and optionally a cast copy of x); MODE 1: out = silu(y)
 //   conv_hist_update  the slot's history after the step: the last taps-1 inputs of old history ++ this step's rows
-//   delta_rule        gated delta rule, one wave per (item, head, 64 value columns), a state column per lane:
+//   delta_rule        gated delta rule, one wave per (item, head, 16 value columns), a quarter state column per lane:
 //                       S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
 //                     q, k made unit vectors per head (1e-6 inside the root), q times D^-1/2;
 //                     beta = sigmoid(b), g = exp(-exp(A_log) softplus(a + dt_bias)); state fp32 [slot][H][D][Dv]
@@ -76,74 +76,94 @@ __global__ void conv_hist_update_kernel(const IT* __restrict__ x, int ldx, float
   }
 }
 
-// qkv fp32 rows [q (G*D) | k (G*D) | v (H*Dv)]; ba rows hold the beta logits at column b_off and the decay
-// inputs at column a_off, one per head.
-template <typename AT, int DMAX>
-__global__ void __launch_bounds__(64) delta_rule_kernel(const float* __restrict__ qkv, int ldq, const AT* __restrict__ ba,
-                                                         int ldb, int b_off, int a_off, const float* __restrict__ A_log,
-                                                         const float* __restrict__ dt_bias, float* __restrict__ state,
-                                                         long long slot_stride, const int* __restrict__ cu,
-                                                         const int* __restrict__ item_slot,
+// Before the recurrence, per row and in parallel over rows: q and k (fp32 rows [q (G*D) | k (G*D) | v (H*Dv)]) made
+// unit vectors per head IN PLACE (q also times D^-1/2), and bg[t] = [beta_h | decay_h] from the projection columns
+// ba[:, b_off + h], ba[:, a_off + h].
+template <typename AT>
+__global__ void delta_prep_kernel(float* __restrict__ qkv, int ldq, const AT* __restrict__ ba, int ldb, int b_off,
+                                  int a_off, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
+                                  float* __restrict__ bg, int H, int G, int D) {
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const float qscale = 1.0f / sqrtf((float)D);
+  for (int v = wv; v < 2 * G; v += nw) {  // q heads, then k heads
+    float* x = qkv + (size_t)t * ldq + (size_t)v * D;
+    float s = 0.f;
+    for (int i = lane; i < D; i += 64) s += x[i] * x[i];
+    const float r = (v < G ? qscale : 1.0f) / sqrtf(wave_sum(s) + 1e-6f);
+    for (int i = lane; i < D; i += 64) x[i] *= r;
+  }
+  for (int h = threadIdx.x; h < H; h += blockDim.x) {
+    bg[(size_t)t * 2 * H + h] = sigmoid_f(Elem<AT>::ld(ba + (size_t)t * ldb + b_off + h));
+    bg[(size_t)t * 2 * H + H + h] = expf(-expf(A_log[h]) * softplus_f(Elem<AT>::ld(ba + (size_t)t * ldb + a_off + h) + dt_bias[h]));
+  }
+}
+
+// The recurrence: one wave per (item, head, 16 value columns); lane = 16 r + c holds rows [r DPL, (r + 1) DPL) of
+// state column c, so a token costs D / 4 multiply-adds per lane for each of the two dot products and the two
+// updates, and the partial dot products meet through two lane swaps.  The next token's operands are loaded while
+// the current one is computed.
+template <int DPL>
+__global__ void __launch_bounds__(64) delta_rule_kernel(const float* __restrict__ qkv, int ldq, const float* __restrict__ bg,
+                                                         float* __restrict__ state, long long slot_stride,
+                                                         const int* __restrict__ cu, const int* __restrict__ item_slot,
                                                          const int* __restrict__ positions, float* __restrict__ out,
                                                          int ldo, int H, int G, int D, int Dv, int tiles) {
-  __shared__ float ks[DMAX], qs[DMAX];
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x, c = lane & 15, r = lane >> 4;
   const int item = blockIdx.y, h = blockIdx.x / tiles, tile = blockIdx.x - h * tiles;
-  const int col = tile * 64 + lane;
+  const int col = tile * 16 + c;
   const bool live = col < Dv;
   const int kvh = h / (H / G);
   const int r0 = cu[item], r1 = cu[item + 1];
   if (r1 <= r0) return;
-  float* Sg = state + (long long)item_slot[item] * slot_stride + ((size_t)h * D) * Dv + col;
-  float S[DMAX];
+  const int i0 = r * DPL;  // this lane's first state row
+  float* Sg = state + (long long)item_slot[item] * slot_stride + ((size_t)h * D + i0) * Dv + col;
+  float S[DPL];
   const bool fresh = positions[r0] == 0;
 #pragma unroll
-  for (int i = 0; i < DMAX; ++i) S[i] = (i < D && live && !fresh) ? Sg[(size_t)i * Dv] : 0.f;
-  const float nA = -expf(A_log[h]), dtb = dt_bias[h];
-  const float qscale = 1.0f / sqrtf((float)D);
+  for (int j = 0; j < DPL; ++j) S[j] = (i0 + j < D && live && !fresh) ? Sg[(size_t)j * Dv] : 0.f;
   const int nq = G * D;
-  for (int row = r0; row < r1; ++row) {
-    const float* qr = qkv + (size_t)row * ldq + kvh * D;
+  float kq[2][2 * DPL];  // [buffer][k rows | q rows]
+  float vb[2], bb[2], gb[2];
+  auto fetch = [&](int row, int buf) {
+    const float* qr = qkv + (size_t)row * ldq + kvh * D + i0;
     const float* kr = qr + nq;
-    float sq = 0.f, sk = 0.f;
-    for (int i = lane; i < D; i += 64) {
-      const float a = qr[i], b = kr[i];
-      sq += a * a;
-      sk += b * b;
+#pragma unroll
+    for (int j = 0; j < DPL; ++j) {
+      const bool ok = i0 + j < D;
+      kq[buf][j] = ok ? kr[j] : 0.f;
+      kq[buf][DPL + j] = ok ? qr[j] : 0.f;
     }
-    sq = wave_sum(sq);
-    sk = wave_sum(sk);
-    const float rq = qscale / sqrtf(sq + 1e-6f), rk = 1.0f / sqrtf(sk + 1e-6f);
-    __syncthreads();
-    for (int i = lane; i < D; i += 64) {
-      qs[i] = qr[i] * rq;
-      ks[i] = kr[i] * rk;
-    }
-    __syncthreads();
-    const float v = live ? qkv[(size_t)row * ldq + 2 * nq + h * Dv + col] : 0.f;
-    const float beta = sigmoid_f(Elem<AT>::ld(ba + (size_t)row * ldb + b_off + h));
-    const float g = expf(nA * softplus_f(Elem<AT>::ld(ba + (size_t)row * ldb + a_off + h) + dtb));
+    vb[buf] = live ? qkv[(size_t)row * ldq + 2 * nq + h * Dv + col] : 0.f;
+    bb[buf] = bg[(size_t)row * 2 * H + h];
+    gb[buf] = bg[(size_t)row * 2 * H + H + h];
+  };
+  fetch(r0, 0);
+  for (int row = r0; row < r1; ++row) {
+    const int cur = (row - r0) & 1;
+    if (row + 1 < r1) fetch(row + 1, cur ^ 1);
+    const float g = gb[cur];
     float dot = 0.f;
 #pragma unroll
-    for (int i = 0; i < DMAX; ++i)
-      if (i < D) {
-        S[i] *= g;
-        dot += S[i] * ks[i];
-      }
-    const float u = beta * (v - dot);
+    for (int j = 0; j < DPL; ++j) {
+      S[j] *= g;
+      dot += S[j] * kq[cur][j];
+    }
+    dot = row_sum4(dot);
+    const float u = bb[cur] * (vb[cur] - dot);
     float o = 0.f;
 #pragma unroll
-    for (int i = 0; i < DMAX; ++i)
-      if (i < D) {
-        S[i] += ks[i] * u;
-        o += S[i] * qs[i];
-      }
-    if (live) out[(size_t)row * ldo + h * Dv + col] = o;
+    for (int j = 0; j < DPL; ++j) {
+      S[j] += kq[cur][j] * u;
+      o += S[j] * kq[cur][DPL + j];
+    }
+    o = row_sum4(o);
+    if (live && r == 0) out[(size_t)row * ldo + h * Dv + col] = o;
   }
   if (live) {
 #pragma unroll
-    for (int i = 0; i < DMAX; ++i)
-      if (i < D) Sg[(size_t)i * Dv] = S[i];
+    for (int j = 0; j < DPL; ++j)
+      if (i0 + j < D) Sg[(size_t)j * Dv] = S[j];
   }
 }
 
@@ -214,26 +234,24 @@ extern "C" int r32_conv_hist_update(const void* x, int ldx, float* hist, long lo
 
 extern "C" int r32_delta_rule_max_dim() { return 256; }
 
-extern "C" int r32_delta_rule(const float* qkv, int ldq, const void* ba, int ldb, int b_off, int a_off, const float* A_log,
-                              const float* dt_bias, float* state, long long slot_stride, const int* cu,
-                              const int* item_slot, const int* positions, float* out, int ldo, int items, int H, int G,
-                              int D, int Dv, int f32, hipStream_t s) {
-  if (items <= 0) return 0;
+// qkv is normalised in place (q, k columns); bg fp32 [T, 2 H] scratch for beta and the decays
+extern "C" int r32_delta_rule(float* qkv, int ldq, const void* ba, int ldb, int b_off, int a_off, const float* A_log,
+                              const float* dt_bias, float* bg, float* state, long long slot_stride, const int* cu,
+                              const int* item_slot, const int* positions, float* out, int ldo, int T, int items, int H,
+                              int G, int D, int Dv, int f32, hipStream_t s) {
+  if (items <= 0 || T <= 0) return 0;
   if (D < 1 || D > 256 || H % G != 0) return -1;
-  const int tiles = (Dv + 63) / 64;
+  if (f32) delta_prep_kernel<float><<<T, 256, 0, s>>>(qkv, ldq, (const float*)ba, ldb, b_off, a_off, A_log, dt_bias, bg, H, G, D);
+  else delta_prep_kernel<bf16_t><<<T, 256, 0, s>>>(qkv, ldq, (const bf16_t*)ba, ldb, b_off, a_off, A_log, dt_bias, bg, H, G, D);
+  const int tiles = (Dv + 15) / 16;
   dim3 grid(H * tiles, items);
-#define LWC_DELTA(AT, DM)                                                                                              \
-  delta_rule_kernel<AT, DM><<<grid, 64, 0, s>>>(qkv, ldq, (const AT*)ba, ldb, b_off, a_off, A_log, dt_bias, state,    \
-                                                slot_stride, cu, item_slot, positions, out, ldo, H, G, D, Dv, tiles)
-  if (f32) {
-    if (D <= 64) LWC_DELTA(float, 64);
-    else if (D <= 128) LWC_DELTA(float, 128);
-    else LWC_DELTA(float, 256);
-  } else {
-    if (D <= 64) LWC_DELTA(bf16_t, 64);
-    else if (D <= 128) LWC_DELTA(bf16_t, 128);
-    else LWC_DELTA(bf16_t, 256);
-  }
+#define LWC_DELTA(DPL)                                                                                             \
+  delta_rule_kernel<DPL><<<grid, 64, 0, s>>>(qkv, ldq, bg, state, slot_stride, cu, item_slot, positions, out, ldo, \
+                                             H, G, D, Dv, tiles)
+  if (D <= 32) LWC_DELTA(8);
+  else if (D <= 64) LWC_DELTA(16);
+  else if (D <= 128) LWC_DELTA(32);
+  else LWC_DELTA(64);
 #undef LWC_DELTA
   LWC_CHECK_LAUNCH();
   return 0;

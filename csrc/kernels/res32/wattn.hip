@@ -202,7 +202,7 @@ struct WAttnMfmaParams {
   int tiles_per_item;
   const int* block_tables;
   int bt_width;
-  const float* bias;  // [H, window]
+  const float* bias;  // [H, window], or null: no distance bias
   int window;
   bf16_t* out;
   int ldo, H, G;
@@ -260,7 +260,7 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
 #pragma unroll
   for (int n = 0; n < NV; ++n) O[n] = float4v{0.f, 0.f, 0.f, 0.f};
   float m = -1e30f, l = 0.f;
-  const float* bias_h = p.bias + (size_t)h * p.window;
+  const float* bias_h = p.bias ? p.bias + (size_t)h * p.window : nullptr;  // no table: no distance bias
 
   const int pg0 = page_ix((j_lo / 32) * 32);  // first page of the workgroup's key range
   // a tile's words are fetched into registers one tile ahead (the loads fly while the previous tile is computed)
@@ -293,7 +293,7 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
     }
     if (tid < 96) {
       const int dist = pos0 - kt * 32 - 31 + tid;  // (row - key + 31) = tid
-      breg = dist >= 0 && dist < p.window ? bias_h[dist] * kLog2e : 0.f;  // the softmax runs in the log2 domain
+      breg = bias_h && dist >= 0 && dist < p.window ? bias_h[dist] * kLog2e : 0.f;  // the softmax runs in the log2 domain
     }
   };
   auto stash = [&](int buf) {

@@ -29,7 +29,7 @@ struct WAttnDecodeParams {
   const int* positions;    // [B]: the new token's position (its key is already in the cache)
   const int* block_tables;
   int bt_width;
-  const float* bias;       // [H, window]
+  const float* bias;       // [H, window], or null: no distance bias
   int window;
   float* part_o;           // [B, H, S, Dv]
   float* part_ml;          // [B, H, S, 2]
@@ -78,7 +78,7 @@ __global__ void __launch_bounds__(64) window_attn_decode_kernel(const WAttnDecod
 #pragma unroll
   for (int n = 0; n < NV; ++n) O[n] = float4v{0.f, 0.f, 0.f, 0.f};
   float m = -1e30f, l = 0.f;
-  const float* bias_h = p.bias + (size_t)h * p.window;
+  const float* bias_h = p.bias ? p.bias + (size_t)h * p.window : nullptr;  // no table: no distance bias
 
   for (int t0 = base; t0 <= last; t0 += 32) {
     float4v sacc[2];
@@ -102,7 +102,7 @@ __global__ void __launch_bounds__(64) window_attn_decode_kernel(const WAttnDecod
       const int j = t0 + (e >> 2) * 16 + 4 * g4 + (e & 3);
       const int dist = i - j;
       ok[e] = h_valid && dist >= 0 && dist < p.window && j <= last;
-      s[e] = ok[e] ? sacc[e >> 2][e & 3] - bias_h[dist] : -1e30f;
+      s[e] = ok[e] ? sacc[e >> 2][e & 3] - (bias_h ? bias_h[dist] : 0.f) : -1e30f;
       mx = fmaxf(mx, s[e]);
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));

@@ -363,7 +363,7 @@ class MerudraModel:
             ci = self.cache_index[li]
             z = self._no_bias(m.heads)
             res32.window_attn(q[rows], cache.k[ci], cache.v[ci], positions[rows], tables, z, z, UNBOUNDED, out[rows],
-                              m.heads, m.kv_heads, cu_q=cu_q, k_lens=k_lens, max_q=max_q, bias=None)
+                              m.heads, m.kv_heads, cu_q=cu_q, k_lens=k_lens, max_q=max_q, bias=None, cores=True)
         return run
 
     def decode(self, tokens: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor, block_tables: torch.Tensor,

@@ -104,15 +104,16 @@ def distance_bias(r1: torch.Tensor, r2: torch.Tensor, window: int) -> torch.Tens
 def window_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, positions: torch.Tensor,
                 block_tables: torch.Tensor, r1: torch.Tensor, r2: torch.Tensor, window: int, out: torch.Tensor,
                 H: int, G: int, cu_q: Optional[torch.Tensor] = None, k_lens: Optional[torch.Tensor] = None,
-                max_q: int = 0, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+                max_q: int = 0, bias: Optional[torch.Tensor] = None, cores: Optional[bool] = None) -> torch.Tensor:
     """Sliding-window attention over the paged cache with the bias -r1_h ln(1 + r2_h (i - j)); ``q`` fp32
     [T, H*D] pre-scaled; row t reads table row t (``cu_q`` None) or the item whose ``cu_q`` range holds t.
     Over a bf16 cache whose sizes the matrix-core kernels are built for, prompt portions run on the portion kernel
     (it wants ``k_lens``, ``max_q`` and the ``bias`` table of :func:`distance_bias`) and decode rows on the
-    split-key decode kernel (``bias``); everything else on the general kernel."""
+    split-key decode kernel (``bias``); everything else on the general kernel.  ``cores=True`` with ``bias`` None:
+    the matrix-core kernels without a distance bias (r1 = 0: plain causal or windowed softmax attention)."""
     K = kernels()
     bs = k_cache.shape[1]
-    cores = (bias is not None and k_cache.dtype == torch.bfloat16 and bs & (bs - 1) == 0
+    cores = ((bias is not None or bool(cores)) and k_cache.dtype == torch.bfloat16 and bs & (bs - 1) == 0
              and K.window_attn_mfma_ok(k_cache.shape[2] // G, v_cache.shape[2] // G))
     if cores and cu_q is None and positions.numel() > 0:
         max_keys = min(int(window), block_tables.shape[1] * k_cache.shape[1])
@@ -165,7 +166,7 @@ def delta_rule(qkv: torch.Tensor, ba: torch.Tensor, b_off: int, a_off: int, A_lo
     """Gated delta rule over a step's items: per head S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q
     with q, k unit vectors per head (q times D^-1/2), beta = sigmoid(ba[:, b_off + h]),
     g = exp(-exp(A_log_h) softplus(ba[:, a_off + h] + dt_bias_h)).  ``qkv`` fp32 [T, 2 G D + H Dv] (after the
-    short convolutions), ``state`` fp32 [slots, H, D, Dv] (read unless the item starts at position 0, written
+    short convolutions; its q and k columns are normalised IN PLACE), ``state`` fp32 [slots, H, D, Dv] (read unless the item starts at position 0, written
     back).  Returns o fp32 [T, H Dv]."""
     if out is None:
         out = torch.empty(qkv.shape[0], H * state.shape[3], dtype=torch.float32, device=qkv.device)
