@@ -99,19 +99,24 @@ __global__ void delta_prep_kernel(float* __restrict__ qkv, int ldq, const AT* __
   }
 }
 
-// The recurrence: one wave per (item, head, 16 value columns); lane = 16 r + c holds rows [r DPL, (r + 1) DPL) of
-// state column c, so a token costs D / 4 multiply-adds per lane for each of the two dot products and the two
-// updates, and the partial dot products meet through two lane swaps.  The next token's operands are loaded while
-// the current one is computed.
-template <int DPL>
-__global__ void __launch_bounds__(64) delta_rule_kernel(const float* __restrict__ qkv, int ldq, const float* __restrict__ bg,
-                                                         float* __restrict__ state, long long slot_stride,
-                                                         const int* __restrict__ cu, const int* __restrict__ item_slot,
-                                                         const int* __restrict__ positions, float* __restrict__ out,
-                                                         int ldo, int H, int G, int D, int Dv, int tiles) {
-  const int lane = threadIdx.x, c = lane & 15, r = lane >> 4;
-  const int item = blockIdx.y, h = blockIdx.x / tiles, tile = blockIdx.x - h * tiles;
-  const int col = tile * 16 + c;
+// The recurrence: a workgroup of NW waves per (item, head, 16 NW value columns), one wave per 16 columns; lane =
+// 16 r + c holds rows [r DPL, (r + 1) DPL) of state column c, so a token costs D / 4 multiply-adds per lane for each
+// of the two dot products and the two updates, and the partial dot products meet through two lane swaps.  A
+// token's k and q (shared by all columns of the head) are staged through LDS, double-buffered: the next token's
+// operands are in flight while the current one is computed, one barrier per token.
+template <int DPL, int NW>
+__global__ void __launch_bounds__(64 * NW) delta_rule_kernel(const float* __restrict__ qkv, int ldq,
+                                                              const float* __restrict__ bg, float* __restrict__ state,
+                                                              long long slot_stride, const int* __restrict__ cu,
+                                                              const int* __restrict__ item_slot,
+                                                              const int* __restrict__ positions, float* __restrict__ out,
+                                                              int ldo, int H, int G, int D, int Dv, int groups) {
+  constexpr int QLD = DPL + 4;               // a quarter's row in LDS, padded against bank conflicts
+  constexpr int PER = (8 * DPL + 64 * NW - 1) / (64 * NW);  // staged floats per thread (k and q: 2 * 4 DPL)
+  __shared__ __attribute__((aligned(16))) float kq_s[2][2][4 * QLD];  // [buffer][k | q][quarter rows]
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, c = lane & 15, r = lane >> 4;
+  const int item = blockIdx.y, h = blockIdx.x / groups, grp = blockIdx.x - h * groups;
+  const int col = (grp * NW + wv) * 16 + c;
   const bool live = col < Dv;
   const int kvh = h / (H / G);
   const int r0 = cu[item], r1 = cu[item + 1];
@@ -123,42 +128,67 @@ __global__ void __launch_bounds__(64) delta_rule_kernel(const float* __restrict_
 #pragma unroll
   for (int j = 0; j < DPL; ++j) S[j] = (i0 + j < D && live && !fresh) ? Sg[(size_t)j * Dv] : 0.f;
   const int nq = G * D;
-  float kq[2][2 * DPL];  // [buffer][k rows | q rows]
-  float vb[2], bb[2], gb[2];
-  auto fetch = [&](int row, int buf) {
-    const float* qr = qkv + (size_t)row * ldq + kvh * D + i0;
-    const float* kr = qr + nq;
+  float stage[PER], vn = 0.f, bn = 0.f, gn = 0.f;
+  auto fetch = [&](int row) {  // the row's k and q chunk of this thread, its value, beta and decay -> registers
+    const float* qr = qkv + (size_t)row * ldq + kvh * D;
 #pragma unroll
-    for (int j = 0; j < DPL; ++j) {
-      const bool ok = i0 + j < D;
-      kq[buf][j] = ok ? kr[j] : 0.f;
-      kq[buf][DPL + j] = ok ? qr[j] : 0.f;
+    for (int u = 0; u < PER; ++u) {
+      const int e = tid + 64 * NW * u;       // e < 4 DPL: k row e; else q row e - 4 DPL
+      const int which = e >= 4 * DPL, i = e - which * 4 * DPL;
+      stage[u] = (e < 8 * DPL && i < D) ? qr[(which ? 0 : nq) + i] : 0.f;
     }
-    vb[buf] = live ? qkv[(size_t)row * ldq + 2 * nq + h * Dv + col] : 0.f;
-    bb[buf] = bg[(size_t)row * 2 * H + h];
-    gb[buf] = bg[(size_t)row * 2 * H + H + h];
+    vn = live ? qkv[(size_t)row * ldq + 2 * nq + h * Dv + col] : 0.f;
+    bn = bg[(size_t)row * 2 * H + h];
+    gn = bg[(size_t)row * 2 * H + H + h];
   };
-  fetch(r0, 0);
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int e = tid + 64 * NW * u;
+      const int which = e >= 4 * DPL, i = e - which * 4 * DPL;
+      if (e < 8 * DPL) kq_s[buf][which][(i / DPL) * QLD + i % DPL] = stage[u];
+    }
+  };
+  fetch(r0);
+  stash(0);
+  float v = vn, beta = bn, g = gn;
+  __syncthreads();
   for (int row = r0; row < r1; ++row) {
     const int cur = (row - r0) & 1;
-    if (row + 1 < r1) fetch(row + 1, cur ^ 1);
-    const float g = gb[cur];
+    if (row + 1 < r1) fetch(row + 1);
+    const float4v* ks = reinterpret_cast<const float4v*>(&kq_s[cur][0][r * QLD]);
+    const float4v* qs = reinterpret_cast<const float4v*>(&kq_s[cur][1][r * QLD]);
+    float kk[DPL];
     float dot = 0.f;
 #pragma unroll
-    for (int j = 0; j < DPL; ++j) {
-      S[j] *= g;
-      dot += S[j] * kq[cur][j];
+    for (int j = 0; j < DPL / 4; ++j) {
+      const float4v k4 = ks[j];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        kk[4 * j + e] = k4[e];
+        S[4 * j + e] *= g;
+        dot += S[4 * j + e] * k4[e];
+      }
     }
     dot = row_sum4(dot);
-    const float u = bb[cur] * (vb[cur] - dot);
+    const float u = beta * (v - dot);
     float o = 0.f;
 #pragma unroll
-    for (int j = 0; j < DPL; ++j) {
-      S[j] += kq[cur][j] * u;
-      o += S[j] * kq[cur][DPL + j];
+    for (int j = 0; j < DPL / 4; ++j) {
+      const float4v q4 = qs[j];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        S[4 * j + e] += kk[4 * j + e] * u;
+        o += S[4 * j + e] * q4[e];
+      }
     }
     o = row_sum4(o);
     if (live && r == 0) out[(size_t)row * ldo + h * Dv + col] = o;
+    if (row + 1 < r1) {
+      stash(cur ^ 1);
+      v = vn, beta = bn, g = gn;
+    }
+    __syncthreads();
   }
   if (live) {
 #pragma unroll
@@ -244,14 +274,27 @@ extern "C" int r32_delta_rule(float* qkv, int ldq, const void* ba, int ldb, int 
   if (f32) delta_prep_kernel<float><<<T, 256, 0, s>>>(qkv, ldq, (const float*)ba, ldb, b_off, a_off, A_log, dt_bias, bg, H, G, D);
   else delta_prep_kernel<bf16_t><<<T, 256, 0, s>>>(qkv, ldq, (const bf16_t*)ba, ldb, b_off, a_off, A_log, dt_bias, bg, H, G, D);
   const int tiles = (Dv + 15) / 16;
-  dim3 grid(H * tiles, items);
-#define LWC_DELTA(DPL)                                                                                             \
-  delta_rule_kernel<DPL><<<grid, 64, 0, s>>>(qkv, ldq, bg, state, slot_stride, cu, item_slot, positions, out, ldo, \
-                                             H, G, D, Dv, tiles)
-  if (D <= 32) LWC_DELTA(8);
-  else if (D <= 64) LWC_DELTA(16);
-  else if (D <= 128) LWC_DELTA(32);
-  else LWC_DELTA(64);
+#define LWC_DELTA(DPL, NW)                                                                                          \
+  delta_rule_kernel<DPL, NW><<<dim3(H * ((tiles + NW - 1) / NW), items), 64 * NW, 0, s>>>(                         \
+      qkv, ldq, bg, state, slot_stride, cu, item_slot, positions, out, ldo, H, G, D, Dv, (tiles + NW - 1) / NW)
+#define LWC_DELTA_NW(DPL)      \
+  if (tiles >= 4) {            \
+    LWC_DELTA(DPL, 4);         \
+  } else if (tiles >= 2) {     \
+    LWC_DELTA(DPL, 2);         \
+  } else {                     \
+    LWC_DELTA(DPL, 1);         \
+  }
+  if (D <= 32) {
+    LWC_DELTA_NW(8)
+  } else if (D <= 64) {
+    LWC_DELTA_NW(16)
+  } else if (D <= 128) {
+    LWC_DELTA_NW(32)
+  } else {
+    LWC_DELTA_NW(64)
+  }
+#undef LWC_DELTA_NW
 #undef LWC_DELTA
   LWC_CHECK_LAUNCH();
   return 0;
