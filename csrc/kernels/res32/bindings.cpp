@@ -24,8 +24,8 @@ int r32_window_attn_mfma(const float*, const void*, const void*, long long, long
 int r32_window_attn_decode_splits(int, int, int, int);
 int r32_window_attn_decode(const float*, const void*, const void*, long long, long long, int, const int*, const int*, int,
                            const float*, int, float*, float*, int, int, void*, int, int, int, int, int, int, hipStream_t);
-int r32_conv_hist(const void*, int, const float*, const float*, long long, const int*, const int*, const int*, const int*,
-                  void*, int, void*, int, int, int, int, int, int, hipStream_t);
+int r32_conv_hist(const void*, int, const float*, int, int, const float*, long long, const int*, const int*, const int*,
+                  const int*, void*, int, void*, int, int, int, int, int, int, hipStream_t);
 int r32_conv_hist_update(const void*, int, float*, long long, const int*, const int*, int, int, int, int, hipStream_t);
 int r32_delta_rule_max_dim();
 int r32_delta_rule(float*, int, const void*, int, int, int, const float*, const float*, float*, float*, long long, const int*,
@@ -319,7 +319,7 @@ void conv_hist(Tensor x, Tensor w, Tensor hist, Tensor row_item, Tensor cu, Tens
                c10::optional<Tensor> out2, int64_t mode) {
   const int fi = act_f32(x, "conv_hist x"), fo = act_f32(out, "conv_hist out");
   const int ldx = row_stride(x, "conv_hist x"), ldo = row_stride(out, "conv_hist out");
-  want(w, torch::kFloat32, "conv_hist w");
+  want_dev(w, torch::kFloat32, "conv_hist w");  // [C, taps], any strides (tap-major storage takes the 16-byte path)
   const int C = (int)x.size(1), taps = (int)w.size(1);
   TORCH_CHECK(w.dim() == 2 && w.size(0) == C && out.size(0) == x.size(0) && out.size(1) == C, "conv_hist: shapes disagree");
   const long long ss = hist_layout(hist, taps, C, "conv_hist hist");
@@ -333,7 +333,8 @@ void conv_hist(Tensor x, Tensor w, Tensor hist, Tensor row_item, Tensor cu, Tens
     ldo2 = row_stride(*out2, "conv_hist out2");
     o2 = out2->data_ptr();
   }
-  done(r32_conv_hist(x.data_ptr(), ldx, w.data_ptr<float>(), hist.data_ptr<float>(), ss, it.row_item, it.cu, it.slot, it.pos,
+  done(r32_conv_hist(x.data_ptr(), ldx, w.data_ptr<float>(), (int)w.stride(0), (int)w.stride(1), hist.data_ptr<float>(), ss,
+                     it.row_item, it.cu, it.slot, it.pos,
                      out.data_ptr(), ldo, o2, ldo2, it.T, C, taps, (int)mode, fi | (fo << 1), stream()), "conv_hist");
 }
 

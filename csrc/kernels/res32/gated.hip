@@ -102,6 +102,45 @@ __global__ void gated_norm_residual_kernel(float* __restrict__ x, const YT* __re
   }
 }
 
+// Rows of d <= 4 * 256 * NCH elements, every base a multiple of four elements: z stays in registers between the sum
+// of squares and the update; 16-byte accesses of x.
+template <typename YT, typename GT, int NCH>
+__global__ void __launch_bounds__(256) gated_norm_residual_vec_kernel(float* __restrict__ x, const YT* __restrict__ y, int ldy,
+                                                                       const GT* __restrict__ r, int ldr,
+                                                                       const float* __restrict__ w,
+                                                                       bf16_t* __restrict__ x_cast, int d, float eps) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  const YT* yr = y + (size_t)t * ldy;
+  const GT* rr = r ? r + (size_t)t * ldr : nullptr;
+  float4v z[NCH];
+  float s = 0.f;
+#pragma unroll
+  for (int u = 0; u < NCH; ++u) {
+    const int i = (threadIdx.x + 256 * u) * 4;
+    z[u] = float4v{0.f, 0.f, 0.f, 0.f};
+    if (i < d) {
+      z[u] = Vec4<YT>::ld(yr + i);
+      if (rr) {
+        const float4v g = Vec4<GT>::ld(rr + i);
+        z[u] *= float4v{sigmoid_f(g[0]), sigmoid_f(g[1]), sigmoid_f(g[2]), sigmoid_f(g[3])};
+      }
+      s += z[u][0] * z[u][0] + z[u][1] * z[u][1] + z[u][2] * z[u][2] + z[u][3] * z[u][3];
+    }
+  }
+  const float rstd = 1.0f / sqrtf(block_sum(s, scratch) / (float)d + eps);
+  float* xr = x + (size_t)t * d;
+#pragma unroll
+  for (int u = 0; u < NCH; ++u) {
+    const int i = (threadIdx.x + 256 * u) * 4;
+    if (i < d) {
+      const float4v v = Vec4<float>::ld(xr + i) + z[u] * rstd * Vec4<float>::ld(w + i);
+      Vec4<float>::st(xr + i, v);
+      if (x_cast) Vec4<bf16_t>::st(x_cast + (size_t)t * d + i, v);
+    }
+  }
+}
+
 template <typename AT>
 __global__ void rmsnorm_rows_kernel(const float* __restrict__ x, const long long* __restrict__ rows,
                                     const float* __restrict__ w, AT* __restrict__ out, int d, float eps) {
@@ -124,6 +163,15 @@ __global__ void gelu_mul_rows_kernel(const AT* __restrict__ z, int ldz, const AT
     int tok = tokens[t];
     tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
     Elem<AT>::st(out + t * n + c, gelu_tanh_f(Elem<AT>::ld(z + t * ldz + c)) * Elem<AT>::ld(table + (size_t)tok * ldt + off + c));
+  }
+}
+
+__global__ void stack_mix_vec_kernel(const float* __restrict__ X, long long plane, const float* __restrict__ coef, int n,
+                                     float* __restrict__ out, long long total4) {
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < total4; e += (long long)gridDim.x * blockDim.x) {
+    float4v s = float4v{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < n; ++j) s += Vec4<float>::ld(X + j * plane + 4 * e) * coef[j];
+    Vec4<float>::st(out + 4 * e, s);
   }
 }
 
@@ -188,6 +236,32 @@ extern "C" int r32_gate_mul(void* a, int lda, const void* g, int ldg, int T, int
 extern "C" int r32_gated_norm_residual(float* x, const void* y, int ldy, const void* r, int ldr, const float* w,
                                        void* x_cast, int T, int d, float eps, int y_f32, int r_f32, hipStream_t s) {
   if (T <= 0) return 0;
+  const bool vec = d % 4 == 0 && d <= 8192 && ldy % 4 == 0 && ldr % 4 == 0 && aligned_to(x, 16) && aligned_to(w, 16) &&
+                   aligned_to(y, y_f32 ? 16 : 8) && aligned_to(r, r_f32 ? 16 : 8) && aligned_to(x_cast, 8);
+  if (vec) {
+    const int nch = (d + 1023) / 1024;
+#define LWC_GNR(YT, GT)                                                                                                  \
+  if (nch <= 1)                                                                                                          \
+    gated_norm_residual_vec_kernel<YT, GT, 1><<<T, 256, 0, s>>>(x, (const YT*)y, ldy, (const GT*)r, ldr, w, (bf16_t*)x_cast, d, eps); \
+  else if (nch <= 2)                                                                                                     \
+    gated_norm_residual_vec_kernel<YT, GT, 2><<<T, 256, 0, s>>>(x, (const YT*)y, ldy, (const GT*)r, ldr, w, (bf16_t*)x_cast, d, eps); \
+  else if (nch <= 4)                                                                                                     \
+    gated_norm_residual_vec_kernel<YT, GT, 4><<<T, 256, 0, s>>>(x, (const YT*)y, ldy, (const GT*)r, ldr, w, (bf16_t*)x_cast, d, eps); \
+  else                                                                                                                   \
+    gated_norm_residual_vec_kernel<YT, GT, 8><<<T, 256, 0, s>>>(x, (const YT*)y, ldy, (const GT*)r, ldr, w, (bf16_t*)x_cast, d, eps)
+    if (y_f32 && (r_f32 || !r)) {
+      LWC_GNR(float, float);
+    } else if (y_f32) {
+      LWC_GNR(float, bf16_t);
+    } else if (!r_f32 || !r) {
+      LWC_GNR(bf16_t, bf16_t);
+    } else {
+      return -1;
+    }
+#undef LWC_GNR
+    LWC_CHECK_LAUNCH();
+    return 0;
+  }
   if (y_f32 && (r_f32 || !r))
     gated_norm_residual_kernel<float, float><<<T, 256, 0, s>>>(x, (const float*)y, ldy, (const float*)r, ldr, w, (bf16_t*)x_cast, d, eps);
   else if (y_f32)
@@ -223,7 +297,10 @@ extern "C" int r32_gelu_mul_rows(const void* z, int ldz, const void* table, int 
 extern "C" int r32_stack_mix(const float* X, long long plane, const float* coef, int n, float* out, long long total,
                              hipStream_t s) {
   if (total <= 0 || n <= 0) return 0;
-  stack_mix_kernel<<<blocks_for(total), 256, 0, s>>>(X, plane, coef, n, out, total);
+  if (total % 4 == 0 && plane % 4 == 0 && aligned_to(X, 16) && aligned_to(out, 16))
+    stack_mix_vec_kernel<<<blocks_for(total / 4), 256, 0, s>>>(X, plane, coef, n, out, total / 4);
+  else
+    stack_mix_kernel<<<blocks_for(total), 256, 0, s>>>(X, plane, coef, n, out, total);
   LWC_CHECK_LAUNCH();
   return 0;
 }

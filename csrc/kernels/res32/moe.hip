@@ -74,6 +74,47 @@ __global__ void router_topk_kernel(const float* __restrict__ z, const float* __r
   }
 }
 
+// Few router outputs (NE <= NMAX): one THREAD per token, the scores in registers.
+template <int NMAX>
+__global__ void router_topk_thread_kernel(const float* __restrict__ z, const float* __restrict__ corr, int NE, int E, int k,
+                                          int* __restrict__ ids, float* __restrict__ wts, int* __restrict__ counts,
+                                          int* __restrict__ rank, int T) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  const float* zr = z + (size_t)t * NE;
+  float v[NMAX], c[NMAX];
+  float m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < NMAX; ++i) {
+    v[i] = i < NE ? zr[i] : -INFINITY;
+    m = fmaxf(m, v[i]);
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < NMAX; ++i) {
+    v[i] = i < NE ? expf(v[i] - m) : 0.f;
+    sum += v[i];
+  }
+#pragma unroll
+  for (int i = 0; i < NMAX; ++i) {
+    v[i] = v[i] / sum;
+    c[i] = i < NE ? v[i] + corr[i] : -INFINITY;
+  }
+  for (int j = 0; j < k; ++j) {
+    float best = -INFINITY, sc = 0.f;
+    int bi = 0;
+#pragma unroll
+    for (int i = 0; i < NMAX; ++i)
+      if (i < NE && c[i] > best) best = c[i], bi = i, sc = v[i];
+#pragma unroll
+    for (int i = 0; i < NMAX; ++i)
+      if (i == bi) c[i] = -INFINITY;
+    ids[(size_t)t * k + j] = bi;
+    wts[(size_t)t * k + j] = sc;
+    rank[(size_t)t * k + j] = bi < E ? atomicAdd(counts + bi, 1) : -1;
+  }
+}
+
 __global__ void router_offsets_kernel(const int* __restrict__ counts, int E, int* __restrict__ row_off) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     int o = 0;
@@ -156,6 +197,22 @@ __global__ void moe_combine_kernel(const YT* __restrict__ Y, const int* __restri
   }
 }
 
+// four columns per thread (d a multiple of four, aligned bases)
+template <typename AT, typename YT>
+__global__ void moe_combine_vec_kernel(const YT* __restrict__ Y, const int* __restrict__ inv, const float* __restrict__ wts,
+                                       const AT* __restrict__ h, int ldh, int k, float* __restrict__ out, int d) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x * 4; c < d; c += blockDim.x * 4) {
+    float4v s = float4v{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < k; ++j) {
+      const int r = inv[(size_t)t * k + j];
+      const float4v v = r >= 0 ? Vec4<YT>::ld(Y + (size_t)r * d + c) : Vec4<AT>::ld(h + (size_t)t * ldh + c);
+      s += v * wts[(size_t)t * k + j];
+    }
+    Vec4<float>::st(out + (size_t)t * d + c, s);
+  }
+}
+
 }  // namespace
 }  // namespace lwc
 
@@ -168,7 +225,8 @@ extern "C" int r32_router(const float* z, const float* corr, int T, int NE, int 
                           int* rank, int* row_off, int* src, int* row_expert, int* inv, hipStream_t s) {
   if (T <= 0) return 0;
   if (NE > 64 * kMaxPerLane || k < 1 || k > NE || E > NE) return -1;
-  if (NE <= 64) router_topk_kernel<1><<<(T + 3) / 4, 256, 0, s>>>(z, corr, NE, E, k, ids, wts, counts, rank, T);
+  if (NE <= 16) router_topk_thread_kernel<16><<<(T + 63) / 64, 64, 0, s>>>(z, corr, NE, E, k, ids, wts, counts, rank, T);
+  else if (NE <= 64) router_topk_kernel<1><<<(T + 3) / 4, 256, 0, s>>>(z, corr, NE, E, k, ids, wts, counts, rank, T);
   else router_topk_kernel<kMaxPerLane><<<(T + 3) / 4, 256, 0, s>>>(z, corr, NE, E, k, ids, wts, counts, rank, T);
   router_offsets_kernel<<<1, 64, 0, s>>>(counts, E, row_off);
   const int total = T * k;
@@ -196,6 +254,18 @@ extern "C" int r32_expert_rows(const void* h, int ldh, const int* src, const int
 extern "C" int r32_moe_combine(const void* Y, int y_f32, const int* inv, const float* wts, const void* h, int ldh, int T,
                                int k, float* out, int d, int f32, hipStream_t s) {
   if (T <= 0) return 0;
+  if (d % 4 == 0 && ldh % 4 == 0 && aligned_to(Y, y_f32 ? 16 : 8) && aligned_to(h, f32 ? 16 : 8) && aligned_to(out, 16)) {
+    if (f32 && y_f32)
+      moe_combine_vec_kernel<float, float><<<T, 256, 0, s>>>((const float*)Y, inv, wts, (const float*)h, ldh, k, out, d);
+    else if (!f32 && y_f32)
+      moe_combine_vec_kernel<bf16_t, float><<<T, 256, 0, s>>>((const float*)Y, inv, wts, (const bf16_t*)h, ldh, k, out, d);
+    else if (!f32 && !y_f32)
+      moe_combine_vec_kernel<bf16_t, bf16_t><<<T, 256, 0, s>>>((const bf16_t*)Y, inv, wts, (const bf16_t*)h, ldh, k, out, d);
+    else
+      return -1;
+    LWC_CHECK_LAUNCH();
+    return 0;
+  }
   if (f32 && y_f32)
     moe_combine_kernel<float, float><<<T, 256, 0, s>>>((const float*)Y, inv, wts, (const float*)h, ldh, k, out, d);
   else if (!f32 && y_f32)

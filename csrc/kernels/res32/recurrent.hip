@@ -19,7 +19,7 @@ namespace lwc {
 namespace {
 
 template <typename IT, typename OT, int MODE>
-__global__ void conv_hist_kernel(const IT* __restrict__ x, int ldx, const float* __restrict__ w,
+__global__ void conv_hist_kernel(const IT* __restrict__ x, int ldx, const float* __restrict__ w, int ws_c, int ws_j,
                                  const float* __restrict__ hist, long long slot_stride, const int* __restrict__ row_item,
                                  const int* __restrict__ cu, const int* __restrict__ item_slot,
                                  const int* __restrict__ positions, OT* __restrict__ out, int ldo, OT* __restrict__ out2,
@@ -31,18 +31,47 @@ __global__ void conv_hist_kernel(const IT* __restrict__ x, int ldx, const float*
   const int r = t - cu[i], p = positions[t];
   const float* h = hist + (long long)item_slot[i] * slot_stride;
   const float cur = Elem<IT>::ld(x + (size_t)t * ldx + c);
-  float acc = w[(size_t)c * taps + taps - 1] * cur;
+  float acc = w[(size_t)c * ws_c + (size_t)(taps - 1) * ws_j] * cur;
   for (int s = 1; s < taps; ++s) {
     float v = 0.f;
     if (s <= r) v = Elem<IT>::ld(x + (size_t)(t - s) * ldx + c);
     else if (s <= p) v = h[(size_t)(taps - 1 - (s - r)) * C + c];
-    acc += w[(size_t)c * taps + taps - 1 - s] * v;
+    acc += w[(size_t)c * ws_c + (size_t)(taps - 1 - s) * ws_j] * v;
   }
   if (MODE == 0) {
     Elem<OT>::st(out + (size_t)t * ldo + c, cur + acc);
     if (out2) Elem<OT>::st(out2 + (size_t)t * ldo2 + c, cur);
   } else {
     Elem<OT>::st(out + (size_t)t * ldo + c, silu_f(acc));
+  }
+}
+
+// Four channels per thread: weights stored tap-major (w[j][c]), every row base a multiple of four channels.
+template <typename IT, typename OT, int MODE>
+__global__ void conv_hist_vec_kernel(const IT* __restrict__ x, int ldx, const float* __restrict__ w,
+                                     const float* __restrict__ hist, long long slot_stride,
+                                     const int* __restrict__ row_item, const int* __restrict__ cu,
+                                     const int* __restrict__ item_slot, const int* __restrict__ positions,
+                                     OT* __restrict__ out, int ldo, OT* __restrict__ out2, int ldo2, int C, int taps) {
+  const int t = blockIdx.y;
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (c >= C) return;
+  const int i = row_item[t];
+  const int r = t - cu[i], p = positions[t];
+  const float* h = hist + (long long)item_slot[i] * slot_stride;
+  const float4v cur = Vec4<IT>::ld(x + (size_t)t * ldx + c);
+  float4v acc = Vec4<float>::ld(w + (size_t)(taps - 1) * C + c) * cur;
+  for (int s = 1; s < taps; ++s) {
+    float4v v = float4v{0.f, 0.f, 0.f, 0.f};
+    if (s <= r) v = Vec4<IT>::ld(x + (size_t)(t - s) * ldx + c);
+    else if (s <= p) v = Vec4<float>::ld(h + (size_t)(taps - 1 - (s - r)) * C + c);
+    acc += Vec4<float>::ld(w + (size_t)(taps - 1 - s) * C + c) * v;
+  }
+  if (MODE == 0) {
+    Vec4<OT>::st(out + (size_t)t * ldo + c, cur + acc);
+    if (out2) Vec4<OT>::st(out2 + (size_t)t * ldo2 + c, cur);
+  } else {
+    Vec4<OT>::st(out + (size_t)t * ldo + c, float4v{silu_f(acc[0]), silu_f(acc[1]), silu_f(acc[2]), silu_f(acc[3])});
   }
 }
 
@@ -226,25 +255,48 @@ __global__ void head_norm_gate_kernel(const float* __restrict__ o, int ldi, cons
 using namespace lwc;
 
 // io: bit 0 = input fp32 (else bf16), bit 1 = output fp32 (else bf16)
-extern "C" int r32_conv_hist(const void* x, int ldx, const float* w, const float* hist, long long slot_stride,
-                             const int* row_item, const int* cu, const int* item_slot, const int* positions, void* out,
-                             int ldo, void* out2, int ldo2, int T, int C, int taps, int mode, int io, hipStream_t s) {
+// w: element (c, j) at w[c * ws_c + j * ws_j]
+extern "C" int r32_conv_hist(const void* x, int ldx, const float* w, int ws_c, int ws_j, const float* hist,
+                             long long slot_stride, const int* row_item, const int* cu, const int* item_slot,
+                             const int* positions, void* out, int ldo, void* out2, int ldo2, int T, int C, int taps,
+                             int mode, int io, hipStream_t s) {
   if (T <= 0 || C <= 0) return 0;
   if (taps < 1 || taps > kMaxTaps) return -1;
-  dim3 grid((C + 255) / 256, T);
-#define LWC_CONV(IT, OT, M)                                                                                          \
-  conv_hist_kernel<IT, OT, M><<<grid, 256, 0, s>>>((const IT*)x, ldx, w, hist, slot_stride, row_item, cu, item_slot, \
-                                                   positions, (OT*)out, ldo, (OT*)out2, ldo2, C, taps)
+  const int ib = (io & 1) ? 16 : 8, ob = (io & 2) ? 16 : 8;
+  const bool vec = ws_c == 1 && (taps == 1 || ws_j == C) && C % 4 == 0 && ldx % 4 == 0 && ldo % 4 == 0 && ldo2 % 4 == 0 &&
+                   slot_stride % 4 == 0 && aligned_to(x, ib) && aligned_to(out, ob) && aligned_to(out2, ob) &&
+                   aligned_to(w, 16) && aligned_to(hist, 16);
+  dim3 grid(vec ? (C / 4 + 63) / 64 : (C + 255) / 256, T);
+  const int threads = vec ? 64 : 256;
+#define LWC_CONV(IT, OT, M)                                                                                            \
+  if (vec)                                                                                                             \
+    conv_hist_vec_kernel<IT, OT, M><<<grid, threads, 0, s>>>((const IT*)x, ldx, w, hist, slot_stride, row_item, cu,   \
+                                                             item_slot, positions, (OT*)out, ldo, (OT*)out2, ldo2, C, \
+                                                             taps);                                                    \
+  else                                                                                                                 \
+    conv_hist_kernel<IT, OT, M><<<grid, threads, 0, s>>>((const IT*)x, ldx, w, ws_c, ws_j, hist, slot_stride,         \
+                                                         row_item, cu, item_slot, positions, (OT*)out, ldo,            \
+                                                         (OT*)out2, ldo2, C, taps)
   if (mode == 0) {
-    if (io == 3) LWC_CONV(float, float, 0);
-    else if (io == 1) LWC_CONV(float, bf16_t, 0);
-    else if (io == 0) LWC_CONV(bf16_t, bf16_t, 0);
-    else return -1;
+    if (io == 3) {
+      LWC_CONV(float, float, 0);
+    } else if (io == 1) {
+      LWC_CONV(float, bf16_t, 0);
+    } else if (io == 0) {
+      LWC_CONV(bf16_t, bf16_t, 0);
+    } else {
+      return -1;
+    }
   } else {
-    if (io == 3) LWC_CONV(float, float, 1);
-    else if (io == 2) LWC_CONV(bf16_t, float, 1);
-    else if (io == 0) LWC_CONV(bf16_t, bf16_t, 1);
-    else return -1;
+    if (io == 3) {
+      LWC_CONV(float, float, 1);
+    } else if (io == 2) {
+      LWC_CONV(bf16_t, float, 1);
+    } else if (io == 0) {
+      LWC_CONV(bf16_t, bf16_t, 1);
+    } else {
+      return -1;
+    }
   }
 #undef LWC_CONV
   LWC_CHECK_LAUNCH();

@@ -188,6 +188,10 @@ class MerudraModel:
         def f32(name):
             return sd[name].to(device=dev, dtype=torch.float32).contiguous()
 
+        def taps_major(w):
+            """[C, taps] convolution weights stored tap-major (the kernels' 16-byte path reads w[j][c : c + 4])."""
+            return w.t().contiguous().t()
+
         self.embed, self.side_embed = t("embed"), t("side.embed")
         self.final_w, self.head = f32("final.norm"), t("head")
         self.layers: List[MerudraLayer] = []
@@ -201,7 +205,7 @@ class MerudraModel:
                 w_in = torch.cat([t(p + "mix.q"), t(p + "mix.k"), t(p + "mix.v"), t(p + "mix.b"), t(p + "mix.a"),
                                   t(p + "mix.g")], 0).contiguous()
                 b_in = None
-                extra["conv"] = torch.cat([f32(p + "mix.q.conv"), f32(p + "mix.k.conv"), f32(p + "mix.v.conv")], 0).contiguous()
+                extra["conv"] = taps_major(torch.cat([f32(p + "mix.q.conv"), f32(p + "mix.k.conv"), f32(p + "mix.v.conv")], 0))
                 extra["A_log"], extra["dt_bias"], extra["norm"] = f32(p + "mix.A_log"), f32(p + "mix.dt_bias"), f32(p + "mix.norm")
             if L.mlp is not None:
                 e = L.mlp
@@ -215,7 +219,7 @@ class MerudraModel:
                     extra["w_down"] = torch.zeros(0, cfg.hidden, e.ff, dtype=dt, device=dev)
             has = L.mlp is not None
             self.layers.append(MerudraLayer(
-                canon1=f32(p + "canon1"), canon2=f32(p + "canon2") if has else None, w_rg1=t(p + "rg1"), b_rg1=t(p + "rg1.b"),
+                canon1=taps_major(f32(p + "canon1")), canon2=taps_major(f32(p + "canon2")) if has else None, w_rg1=t(p + "rg1"), b_rg1=t(p + "rg1.b"),
                 w_rg2=t(p + "rg2") if has else None, b_rg2=t(p + "rg2.b") if has else None, w_in=w_in, b_in=b_in,
                 w_o=t(p + "mix.o"), norm1=f32(p + "norm1"), norm2=f32(p + "norm2") if has else None,
                 side_gate=t(p + "side.gate"), side_proj=t(p + "side.proj"), side_norm=f32(p + "side.norm"),

@@ -35,16 +35,18 @@ def _items(lens, slots, starts, gpu):
 
 # ------------------------------------------------------------------ mechanisms, one by one
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 3e-2)])
-@pytest.mark.parametrize("taps", [1, 2, 4])
-def test_conv_with_history_in_portions(gpu, dtype, tol, taps):
+@pytest.mark.parametrize("taps,C,tap_major", [(1, 37, False), (2, 37, False), (4, 37, True), (4, 40, True), (3, 264, True)])
+def test_conv_with_history_in_portions(gpu, dtype, tol, taps, C, tap_major):
     """x + conv(x) and silu(conv(x)): two sequences cut into portions (one shorter than the history, single rows,
     the two interleaved in one step) in slots that held other data before, against the whole-sequence oracle."""
     from llm_weighted_consensus_amd.ops import res32
 
     g = torch.Generator().manual_seed(taps)
-    C, na, nb = 37, 23, 9
+    na, nb = 23, 9
     xa, xb = torch.randn(na, C, generator=g).to(dtype), torch.randn(nb, C, generator=g).to(dtype)
     w = torch.randn(C, taps, generator=g)
+    # tap-major storage with a width that is a multiple of four takes the 16-byte kernel
+    wg = w.to(gpu).t().contiguous().t() if tap_major else w.to(gpu)
     hist = torch.randn(4, taps - 1, C, generator=g).to(gpu) * 50  # stale contents of earlier sequences
     for mode in (0, 1):
         ya, yb = O.causal_conv(xa.double(), w.double()), O.causal_conv(xb.double(), w.double())
@@ -57,7 +59,7 @@ def test_conv_with_history_in_portions(gpu, dtype, tol, taps):
             items = _items([n for _, n in step], [slot[k] for k, _ in step], [at[k] for k, _ in step], gpu)
             out = torch.empty(x.shape[0], C, dtype=dtype, device=gpu)
             out2 = torch.empty_like(out) if mode == 0 and dtype == torch.bfloat16 else None
-            res32.conv_hist(x, w.to(gpu), hist, items, out, mode=mode, out2=out2)
+            res32.conv_hist(x, wg, hist, items, out, mode=mode, out2=out2)
             if out2 is not None:
                 assert torch.equal(out2, x)
             o = 0
@@ -135,6 +137,13 @@ def test_head_norm_gate_and_gated_norm_residual(gpu, dtype, tol):
     xg = x.to(gpu)
     res32.gated_norm_residual(xg, y.float().to(gpu), wn.to(gpu), 1e-4)  # fp32 result, no gate
     assert (xg.cpu().double() - (x.double() + O.rms_unit(y.double(), 1e-4) * wn.double())).abs().max() < 1e-5
+    for dw in (2320, 1030):  # several 16-byte chunks per thread; a width the 16-byte kernel does not take
+        xw, yw, rw = torch.randn(3, dw, generator=g), torch.randn(3, dw, generator=g).to(dtype), torch.randn(3, dw, generator=g).to(dtype)
+        ww = 1 + 0.2 * torch.randn(dw, generator=g)
+        xg = xw.to(gpu)
+        res32.gated_norm_residual(xg, yw.to(gpu), ww.to(gpu), 1e-4, gate_logits=rw.to(gpu))
+        ref = xw.double() + O.rms_unit(yw.double() * torch.sigmoid(rw.double()), 1e-4) * ww.double()
+        assert (xg.cpu().double() - ref).abs().max() < 1e-5
     rows = torch.tensor([6, 0, 6, 2], device=gpu)
     n = res32.rmsnorm_rows(x.to(gpu), wn.to(gpu), 1e-4, dtype, rows=rows)
     assert (n.cpu().double() - (O.rms_unit(x.double(), 1e-4) * wn.double())[rows.cpu()]).abs().max() < tol * 6
@@ -239,15 +248,16 @@ def test_far_key_and_page_borders_stand_out(gpu, decode, dtype):
         assert (out[0, D:].cpu().double() - k.double().mean(0)).abs().max() < 0.05
 
 
-def test_router_identity_experts_and_correction(gpu):
+@pytest.mark.parametrize("E,I,top,d", [(5, 3, 3, 24), (30, 10, 4, 24), (90, 10, 6, 23)])
+def test_router_identity_experts_and_correction(gpu, E, I, top, d):
     """The correction moves the choice and not the weight; identity experts return the input; weights are the
     softmax over ALL router outputs, not renormalised; expert-major rows cover every real choice exactly once."""
     from llm_weighted_consensus_amd.ops import res32
 
     g = torch.Generator().manual_seed(8)
-    T, d, E, I, top, ff = 50, 24, 5, 3, 3, 10
+    T, ff = 50, 10
     h = torch.randn(T, d, generator=g)
-    W = {"r.router": torch.randn(E + I, d, generator=g) * 0.6, "r.correction": torch.randn(E + I, generator=g) * 0.3}
+    W = {"r.router": torch.randn(E + I, d, generator=g) * 0.6, "r.correction": torch.randn(E + I, generator=g) * 0.3 / (E + I) * 8}
     for e in range(E):
         W.update({f"r.e{e}.gate": torch.randn(ff, d, generator=g) * 0.3, f"r.e{e}.up": torch.randn(ff, d, generator=g) * 0.3,
                   f"r.e{e}.down": torch.randn(d, ff, generator=g) * 0.3})
