@@ -298,19 +298,24 @@ class MerudraModel:
         return res32.moe_combine(Y, inv, w, h2)
 
     def _forward(self, tokens, positions, slots, cache: PagedLayerCache, state: RecurrentStatePool,
-                 items: res32.StepItems, attend) -> torch.Tensor:
+                 items: res32.StepItems, attend, keep: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Every layer over the step's rows; ``attend(q, li, out)`` runs the attention of layer ``li`` into ``out``.
-        Returns the fp32 stream that the output norm reads, [T, d]."""
+        Returns the fp32 stream that the output norm reads, [T, d].
+
+        ``keep`` (int64 rows): only these rows' final states are wanted (a prompt's last token).  The LAST layer
+        then still runs its mixer and both input convolutions on every row (keys, values, the recurrent state and
+        the convolutions' histories are what later steps read), but the gate, the routed experts, the token input
+        and the layer mix on the kept rows only; returns [len(keep), d]."""
         cfg, dt = self.cfg, self.dtype
         T, d, eps, nl = tokens.shape[0], cfg.hidden, cfg.norm_eps, len(self.layers)
         exact = dt == torch.float32
         X = torch.empty(nl + 1, T, d, dtype=torch.float32, device=self.device)  # every layer's result stays resident
         res32.embed_rows(self.embed, tokens, X[0])
         X[1].copy_(X[0])
-        final = torch.empty(T, d, dtype=torch.float32, device=self.device)
         xb = None if exact else torch.empty(T, d, dtype=dt, device=self.device)
         for li, (S, L) in enumerate(zip(cfg.layer_specs, self.layers)):
             m, x = S.mixer, X[li + 1]
+            short = keep is not None and li + 1 == nl
             h = torch.empty(T, d, dtype=dt, device=self.device)
             res32.conv_hist(x, L.canon1, state[f"c1.{li}"], items, h, mode=0, out2=xb)
             r = self._linear(x if exact else xb, L.w_rg1, L.b_rg1)
@@ -333,15 +338,24 @@ class MerudraModel:
                                       x_cast=xb if S.mlp is None else None)
             if S.mlp is not None:
                 res32.conv_hist(x, L.canon2, state[f"c2.{li}"], items, h, mode=0, out2=xb)
+            toks = tokens
+            if short:  # from here on only the kept rows
+                x, h, toks = x.index_select(0, keep), h.index_select(0, keep), tokens.index_select(0, keep)
+                xb = None if exact else xb.index_select(0, keep)
+            if S.mlp is not None:
                 r = self._linear(x if exact else xb, L.w_rg2, L.b_rg2)
                 res32.gated_norm_residual(x, self._experts(h, L, S.mlp), L.norm2, eps, gate_logits=r, x_cast=xb)
-            g = res32.gelu_mul_rows(self._linear(x if exact else xb, L.side_gate), self.side_embed, li * cfg.side_dim, tokens)
+            g = res32.gelu_mul_rows(self._linear(x if exact else xb, L.side_gate), self.side_embed, li * cfg.side_dim, toks)
             res32.gated_norm_residual(x, self._linear(g, L.side_proj), L.side_norm, eps)
-            nxt = X[li + 2] if li + 1 < nl else final
+            if short:
+                Xk = torch.cat([X[:nl].index_select(1, keep), x[None]], 0)
+                final = torch.empty(keep.numel(), d, dtype=torch.float32, device=self.device)
+                return res32.stack_mix(Xk, L.dwa, nl + 1, final)
+            nxt = X[li + 2] if li + 1 < nl else torch.empty(T, d, dtype=torch.float32, device=self.device)
             res32.stack_mix(X, L.dwa, li + 2, nxt)
             if self.on_layer is not None:
                 self.on_layer(li, nxt)
-        return final
+        return nxt
 
     def _logits(self, x: torch.Tensor, rows: Optional[torch.Tensor], float_logits: bool) -> torch.Tensor:
         h = res32.rmsnorm_rows(x, self.final_w, self.cfg.norm_eps, self.dtype, rows=rows)
@@ -411,8 +425,11 @@ class MerudraModel:
             if chk_run is not None:
                 chk_run(q, li, out, slice(n_dec, T))
 
-        x = self._forward(tokens, positions, slots, cache, state, items, attend)
-        return self._logits(x, logit_rows, float_logits)
+        # prompt portions of which few rows are wanted (a prompt's last token): the last layer's gate, experts and
+        # token input on those rows only
+        keep = logit_rows if n_dec == 0 and self.on_layer is None and 4 * logit_rows.numel() <= T else None
+        x = self._forward(tokens, positions, slots, cache, state, items, attend, keep=keep)
+        return self._logits(x, None if keep is not None else logit_rows, float_logits)
 
     def prefill(self, tokens, positions, slots, cu_seqlens, max_seqlen, last_idx, cache, ctx=None):
         raise RuntimeError("Merudra prefills through forward_mixed over the paged cache (paged_prefill)")

@@ -359,6 +359,23 @@ def test_whole_prompt_and_layers(gpu, tmp_path, name, dtype):
     assert eng.bm.num_free == eng.bm.num_blocks and eng.bm.num_free_state_slots == 4
 
 
+@pytest.mark.parametrize("name,dtype", [("mixed", torch.float32), ("cores", torch.float32), ("odd", torch.float32)])
+def test_few_wanted_rows_and_what_they_leave(gpu, tmp_path, name, dtype):
+    """Portions of which few logits are wanted run the last layer's feed-forward side on those rows only; the logits
+    match, and so do the tokens decoded afterwards from the pages, histories and states those steps left."""
+    cfg, W, model, eng = _build(tmp_path, name, dtype)
+    a, b = _tokens(64, cfg["vocab"], 5), _tokens(37, cfg["vocab"], 6)
+    ra, rb = O.forward(cfg, W, a), O.forward(cfg, W, b)
+    got = eng.step_tokens([("a", a[:50], [49, 3]), ("b", b[:30], [29])])
+    assert _err(got, torch.cat([ra[[49, 3]], rb[[29]]])) < TOL[dtype]
+    got = eng.step_tokens([("a", a[50:60], []), ("b", b[30:], [6])], ["b"])
+    assert _err(got, rb[[36]]) < TOL[dtype]
+    for i in range(60, 64):
+        got = eng.step_tokens([("a", [a[i]], [0])], ["a"] if i == 63 else [])
+        assert _err(got, ra[[i]]) < TOL[dtype]
+    assert eng.bm.num_free == eng.bm.num_blocks and eng.bm.num_free_state_slots == 4
+
+
 @pytest.mark.parametrize("name,dtype", [("mixed", torch.float32), ("odd", torch.float32), ("cores", torch.float32),
                                         ("cores", torch.bfloat16)])
 def test_decode_token_by_token_and_portions(gpu, tmp_path, name, dtype):
