@@ -77,6 +77,19 @@ __global__ void gate_mul_kernel(AT* __restrict__ a, int lda, const AT* __restric
   }
 }
 
+template <typename AT, int MODE>
+__global__ void gate_mul_vec_kernel(AT* __restrict__ a, int lda, const AT* __restrict__ g, int ldg, int n4, long long total4) {
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < total4; e += (long long)gridDim.x * blockDim.x) {
+    const long long r = e / n4;
+    const int c = (int)(e - r * n4) * 4;
+    const float4v z = Vec4<AT>::ld(g + r * ldg + c);
+    AT* p = a + r * lda + c;
+    const float4v m = MODE == 0 ? float4v{sigmoid_f(z[0]), sigmoid_f(z[1]), sigmoid_f(z[2]), sigmoid_f(z[3])}
+                                : float4v{silu_f(z[0]), silu_f(z[1]), silu_f(z[2]), silu_f(z[3])};
+    Vec4<AT>::st(p, Vec4<AT>::ld(p) * m);
+  }
+}
+
 template <typename YT, typename GT>
 __global__ void gated_norm_residual_kernel(float* __restrict__ x, const YT* __restrict__ y, int ldy,
                                            const GT* __restrict__ r, int ldr, const float* __restrict__ w,
@@ -220,6 +233,18 @@ extern "C" int r32_head_norm_kv_write(const void* proj, int ldp, int k_off, int 
 extern "C" int r32_gate_mul(void* a, int lda, const void* g, int ldg, int T, int n, int mode, int f32, hipStream_t s) {
   const long long total = (long long)T * n;
   if (total <= 0) return 0;
+  if (n % 4 == 0 && lda % 4 == 0 && ldg % 4 == 0 && aligned_to(a, f32 ? 16 : 8) && aligned_to(g, f32 ? 16 : 8)) {
+    const int nb4 = blocks_for(total / 4);
+    if (f32) {
+      if (mode == 0) gate_mul_vec_kernel<float, 0><<<nb4, 256, 0, s>>>((float*)a, lda, (const float*)g, ldg, n / 4, total / 4);
+      else gate_mul_vec_kernel<float, 1><<<nb4, 256, 0, s>>>((float*)a, lda, (const float*)g, ldg, n / 4, total / 4);
+    } else {
+      if (mode == 0) gate_mul_vec_kernel<bf16_t, 0><<<nb4, 256, 0, s>>>((bf16_t*)a, lda, (const bf16_t*)g, ldg, n / 4, total / 4);
+      else gate_mul_vec_kernel<bf16_t, 1><<<nb4, 256, 0, s>>>((bf16_t*)a, lda, (const bf16_t*)g, ldg, n / 4, total / 4);
+    }
+    LWC_CHECK_LAUNCH();
+    return 0;
+  }
   const int nb = blocks_for(total);
   if (f32) {
     if (mode == 0) gate_mul_kernel<float, 0><<<nb, 256, 0, s>>>((float*)a, lda, (const float*)g, ldg, n, total);

@@ -79,8 +79,9 @@ template <int NMAX>
 __global__ void router_topk_thread_kernel(const float* __restrict__ z, const float* __restrict__ corr, int NE, int E, int k,
                                           int* __restrict__ ids, float* __restrict__ wts, int* __restrict__ counts,
                                           int* __restrict__ rank, int T) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= T) return;
+  const int t0 = blockIdx.x * blockDim.x + threadIdx.x;
+  const bool live = t0 < T;  // lanes past the last token go along (wave-wide votes below) and write nothing
+  const int t = live ? t0 : T - 1;
   const float* zr = z + (size_t)t * NE;
   float v[NMAX], c[NMAX];
   float m = -INFINITY;
@@ -109,9 +110,23 @@ __global__ void router_topk_thread_kernel(const float* __restrict__ z, const flo
 #pragma unroll
     for (int i = 0; i < NMAX; ++i)
       if (i == bi) c[i] = -INFINITY;
-    ids[(size_t)t * k + j] = bi;
-    wts[(size_t)t * k + j] = sc;
-    rank[(size_t)t * k + j] = bi < E ? atomicAdd(counts + bi, 1) : -1;
+    if (live) {
+      ids[(size_t)t * k + j] = bi;
+      wts[(size_t)t * k + j] = sc;
+    }
+    // one atomic per (wave, expert) instead of one per token: the wave's tokens that chose expert e take
+    // consecutive ranks in lane order
+    int rk = -1;
+    for (int e = 0; e < E; ++e) {
+      const unsigned long long m = __ballot(live && bi == e);
+      if (m == 0ull) continue;
+      const int leader = __ffsll((long long)m) - 1;
+      int base = 0;
+      if ((int)(threadIdx.x & 63) == leader) base = atomicAdd(counts + e, __popcll(m));
+      base = __shfl(base, leader, 64);
+      if (live && bi == e) rk = base + __popcll(m & ((1ull << (threadIdx.x & 63)) - 1ull));
+    }
+    if (live) rank[(size_t)t * k + j] = rk;
   }
 }
 

@@ -249,6 +249,34 @@ __global__ void head_norm_gate_kernel(const float* __restrict__ o, int ldi, cons
   }
 }
 
+// Dv a multiple of four, aligned bases: 16-byte reads of o, four gate values per lane
+template <typename AT, int GATE>
+__global__ void head_norm_gate_vec_kernel(const float* __restrict__ o, int ldi, const AT* __restrict__ gate, int ldg,
+                                          const float* __restrict__ w, AT* __restrict__ out, int ldo, int H, int Dv,
+                                          float eps) {
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  for (int h = wv; h < H; h += nw) {
+    const float* oh = o + (size_t)t * ldi + h * Dv;
+    float s = 0.f;
+    for (int i = lane * 4; i < Dv; i += 256) {
+      const float4v v = Vec4<float>::ld(oh + i);
+      s += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(s) / (float)Dv + eps);
+    for (int i = lane * 4; i < Dv; i += 256) {
+      float4v y = Vec4<float>::ld(oh + i) * rstd;
+      if (w) y *= Vec4<float>::ld(w + i);
+      if (GATE) {
+        const float4v z = Vec4<AT>::ld(gate + (size_t)t * ldg + h * Dv + i);
+        y *= GATE == 1 ? float4v{silu_f(z[0]), silu_f(z[1]), silu_f(z[2]), silu_f(z[3])}
+                       : float4v{sigmoid_f(z[0]), sigmoid_f(z[1]), sigmoid_f(z[2]), sigmoid_f(z[3])};
+      }
+      Vec4<AT>::st(out + (size_t)t * ldo + h * Dv + i, y);
+    }
+  }
+}
+
 }  // namespace
 }  // namespace lwc
 
@@ -356,16 +384,30 @@ extern "C" int r32_head_norm_gate(const float* o, int ldi, const void* gate, int
                                   int T, int H, int Dv, float eps, int gate_mode, int f32, hipStream_t s) {
   if (T <= 0) return 0;
   const int threads = H >= 4 ? 256 : 64 * H;
-#define LWC_HNG(AT, GM)                                                                                           \
-  head_norm_gate_kernel<AT, GM><<<T, threads, 0, s>>>(o, ldi, (const AT*)gate, ldg, w, (AT*)out, ldo, H, Dv, eps)
+  const int ab = f32 ? 16 : 8;
+  const bool vec = Dv % 4 == 0 && ldi % 4 == 0 && ldg % 4 == 0 && ldo % 4 == 0 && aligned_to(o, 16) && aligned_to(w, 16) &&
+                   aligned_to(gate, ab) && aligned_to(out, ab);
+#define LWC_HNG(AT, GM)                                                                                                  \
+  if (vec)                                                                                                               \
+    head_norm_gate_vec_kernel<AT, GM><<<T, threads, 0, s>>>(o, ldi, (const AT*)gate, ldg, w, (AT*)out, ldo, H, Dv, eps); \
+  else                                                                                                                   \
+    head_norm_gate_kernel<AT, GM><<<T, threads, 0, s>>>(o, ldi, (const AT*)gate, ldg, w, (AT*)out, ldo, H, Dv, eps)
   if (f32) {
-    if (gate_mode == 0) LWC_HNG(float, 0);
-    else if (gate_mode == 1) LWC_HNG(float, 1);
-    else LWC_HNG(float, 2);
+    if (gate_mode == 0) {
+      LWC_HNG(float, 0);
+    } else if (gate_mode == 1) {
+      LWC_HNG(float, 1);
+    } else {
+      LWC_HNG(float, 2);
+    }
   } else {
-    if (gate_mode == 0) LWC_HNG(bf16_t, 0);
-    else if (gate_mode == 1) LWC_HNG(bf16_t, 1);
-    else LWC_HNG(bf16_t, 2);
+    if (gate_mode == 0) {
+      LWC_HNG(bf16_t, 0);
+    } else if (gate_mode == 1) {
+      LWC_HNG(bf16_t, 1);
+    } else {
+      LWC_HNG(bf16_t, 2);
+    }
   }
 #undef LWC_HNG
   LWC_CHECK_LAUNCH();

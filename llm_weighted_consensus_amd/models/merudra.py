@@ -96,6 +96,7 @@ class MerudraModel:
                 raise ValueError("Merudra: too many router outputs")
         self.logit_width = -(-cfg.vocab_size // 32) * 32
         self.cache_index = {li: ci for ci, li in enumerate(cfg.attention_layers)}
+        self._mm32 = self._probe_mm32()
         raw = self._read(weights_path) if weights_path else self._random(seed)
         self._assemble(raw)
         self.g8_ws = None
@@ -210,6 +211,10 @@ class MerudraModel:
             if L.mlp is not None:
                 e = L.mlp
                 extra["router"], extra["correction"] = f32(p + "mlp.router"), f32(p + "mlp.correction")
+                if self._mm32 and bool((extra["router"].to(dt).float() == extra["router"]).all()):
+                    extra["router_t"] = extra["router"].to(dt).t().contiguous()
+                else:
+                    self._mm32 = False
                 if e.experts:
                     extra["w_gu"] = torch.stack([torch.cat([t(f"{p}mlp.e{x}.gate"), t(f"{p}mlp.e{x}.up")], 0)
                                                  for x in range(e.experts)]).contiguous()
@@ -226,6 +231,16 @@ class MerudraModel:
                 dwa=f32(p + "dwa"), extra=extra))
 
     # ------------------------------------------------------------------ GEMMs
+    def _probe_mm32(self) -> bool:
+        """Whether this torch build multiplies bf16 matrices into an fp32 result (the router's logits)."""
+        if self.dtype != torch.bfloat16:
+            return False
+        try:
+            a = torch.zeros(8, 16, dtype=self.dtype, device=self.device)
+            return torch.mm(a, a.t(), out_dtype=torch.float32).dtype == torch.float32
+        except (TypeError, RuntimeError):
+            return False
+
     def _linear(self, x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor] = None) -> torch.Tensor:
         if b is None and self.g8_ws is not None:
             return gemm_plan.linear(x, w, ws=self.g8_ws)
@@ -285,7 +300,10 @@ class MerudraModel:
     def _experts(self, h2: torch.Tensor, L: MerudraLayer, e) -> torch.Tensor:
         """Routed experts of the rows h2 -> fp32 [T, d]."""
         x = L.extra
-        z = F.linear(h2.float(), x["router"])  # router logits in fp32
+        if self._mm32:  # bf16 operands, fp32 accumulation AND output: the checkpoint's router is bf16-exact
+            z = torch.mm(h2, x["router_t"], out_dtype=torch.float32)
+        else:
+            z = F.linear(h2.float(), x["router"])  # router logits in fp32
         _ids, w, row_off, src, row_expert, inv = res32.router(z, x["correction"], e.experts, e.top)
         d = self.cfg.hidden
         if (self.dtype == torch.bfloat16 and e.experts and d * e.ff >= self.GROUPED_MIN and d % 64 == 0 and e.ff % 64 == 0

@@ -123,6 +123,10 @@ def test_head_norm_gate_and_gated_norm_residual(gpu, dtype, tol):
     res32.head_norm_gate(o.to(gpu), out, H, 1e-3, w=w.to(gpu), gate=gate.to(gpu)[:, 6:], mode="silu")
     ref = (O.rms_unit(o.double().view(T, H, Dv), 1e-3) * w.double()).reshape(T, -1) * O.silu(gate[:, 6:].double())
     assert (out.cpu().double() - ref).abs().max() < tol * 8
+    gate8 = torch.randn(T, H * Dv + 8, generator=g).to(dtype)  # an offset the 16-byte kernel takes
+    res32.head_norm_gate(o.to(gpu), out, H, 1e-3, w=w.to(gpu), gate=gate8.to(gpu)[:, 8:], mode="sigmoid")
+    ref = (O.rms_unit(o.double().view(T, H, Dv), 1e-3) * w.double()).reshape(T, -1) * torch.sigmoid(gate8[:, 8:].double())
+    assert (out.cpu().double() - ref).abs().max() < tol * 8
     res32.head_norm_gate(o.to(gpu), out, H, 1e-3)
     assert (out.cpu().double() - O.rms_unit(o.double().view(T, H, Dv), 1e-3).reshape(T, -1)).abs().max() < tol * 4
     x = torch.randn(T, d, generator=g) * 4
@@ -167,6 +171,10 @@ def test_embed_side_input_gate_mul_and_stack_mix(gpu, dtype, tol):
     ag = a.to(gpu)
     res32.gate_mul(ag, gt.to(gpu)[:, 19:], "sigmoid")
     assert (ag.cpu().double() - a.double() * torch.sigmoid(gt[:, 19:].double())).abs().max() < tol * 4
+    a, gt = torch.randn(T, 12, generator=g).to(dtype), torch.randn(T, 28, generator=g).to(dtype)  # the 16-byte kernel
+    ag = a.to(gpu)
+    res32.gate_mul(ag, gt.to(gpu)[:, 16:], "silu")
+    assert (ag.cpu().double() - a.double() * O.silu(gt[:, 16:].double())).abs().max() < tol * 4
     X = torch.randn(5, T, d, generator=g)
     coef = torch.randn(4, generator=g)
     Xg = X.to(gpu)
