@@ -309,6 +309,17 @@ CONFIGS = {
 }
 
 
+CONFIGS["recurrent"] = dict(width=36, vocab=90, taps=2, side=4, layers=[  # no attention layer: the paged cache is empty
+    dict(type="delta", heads=2, kv_heads=1, dim=16, vdim=24, conv=2, mlp=None),
+    dict(type="delta", heads=3, kv_heads=3, dim=8, vdim=12, conv=3, mlp=dict(experts=0, identity=3, top=2, ff=8))])
+CONFIGS["attentive"] = dict(width=36, vocab=90, taps=5, side=4, layers=[  # no recurrent layer but the convolutions
+    dict(type="attention", heads=2, kv_heads=1, dim=16, every=2, mlp=dict(experts=6, identity=1, top=6, ff=8)),
+    dict(type="attention", heads=6, kv_heads=3, dim=8, every=50, mlp=None)])
+# experts large enough for the grouped matrix-core GEMMs of the full kernel extension (bf16)
+CONFIGS["grouped"] = dict(width=512, vocab=300, taps=3, side=16, layers=[
+    dict(type="attention", heads=4, kv_heads=2, dim=64, every=16, mlp=dict(experts=4, identity=1, top=2, ff=512))])
+
+
 def _build(tmp_path, name, dtype, seed=0, **engine_kw):
     from safetensors.torch import save_file
 
@@ -349,7 +360,23 @@ def _err(got, ref, dtype=torch.float32):
 TOL = {torch.float32: 3e-4, torch.bfloat16: 0.5}
 
 
-@pytest.mark.parametrize("name", list(CONFIGS))
+def test_grouped_expert_path(gpu, tmp_path):
+    """Experts past the size threshold run through the framework's grouped GEMMs (bf16): a prompt portion and
+    single tokens against the oracle; identity choices and the rows no expert owns do not disturb them."""
+    from llm_weighted_consensus_amd import ops
+
+    assert ops.available()
+    cfg, W, model, eng = _build(tmp_path, "grouped", torch.bfloat16)
+    assert cfg["width"] * cfg["layers"][0]["mlp"]["expert"]["ff"] >= model.GROUPED_MIN
+    toks = _tokens(48, cfg["vocab"], 3)
+    ref = O.forward(cfg, W, toks)
+    got = [eng.step_tokens([("g", toks[:40], list(range(40)))])]
+    for i in range(40, 48):
+        got.append(eng.step_tokens([("g", [toks[i]], [0])], ["g"] if i == 47 else []))
+    assert _err(torch.cat(got), ref, torch.bfloat16) < TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("name", ["mixed", "odd", "cores", "recurrent", "attentive"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_whole_prompt_and_layers(gpu, tmp_path, name, dtype):
     """A whole prompt in one step: the stream after every layer and the logits against the oracle."""
