@@ -24,8 +24,8 @@ int r32_window_attn_mfma(const float*, const void*, const void*, long long, long
 int r32_window_attn_decode_splits(int, int, int, int);
 int r32_window_attn_decode(const float*, const void*, const void*, long long, long long, int, const int*, const int*, int,
                            const float*, int, float*, float*, int, int, void*, int, int, int, int, int, int, hipStream_t);
-int r32_conv_hist(const void*, int, const float*, int, int, const float*, long long, const int*, const int*, const int*,
-                  const int*, void*, int, void*, int, int, int, int, int, int, hipStream_t);
+int r32_conv_hist(const void*, int, const float*, int, int, float*, long long, const int*, const int*, const int*,
+                  const int*, void*, int, void*, int, int, int, int, int, int, int, hipStream_t);
 int r32_conv_hist_update(const void*, int, float*, long long, const int*, const int*, int, int, int, int, hipStream_t);
 int r32_delta_rule_max_dim();
 int r32_delta_rule(float*, int, const void*, int, int, int, const float*, const float*, float*, float*, long long, const int*,
@@ -315,8 +315,9 @@ long long hist_layout(const Tensor& hist, int taps, int C, const char* name) {
 }
 
 // mode 0: out = x + conv(x), out2 (optional) = x in out's dtype; mode 1: out = silu(conv(x)).  w fp32 [C, taps].
+// advance: every item is ONE row (a decode step) and the kernel also moves the slots' histories on.
 void conv_hist(Tensor x, Tensor w, Tensor hist, Tensor row_item, Tensor cu, Tensor item_slot, Tensor positions, Tensor out,
-               c10::optional<Tensor> out2, int64_t mode) {
+               c10::optional<Tensor> out2, int64_t mode, bool advance) {
   const int fi = act_f32(x, "conv_hist x"), fo = act_f32(out, "conv_hist out");
   const int ldx = row_stride(x, "conv_hist x"), ldo = row_stride(out, "conv_hist out");
   want_dev(w, torch::kFloat32, "conv_hist w");  // [C, taps], any strides (tap-major storage takes the 16-byte path)
@@ -325,6 +326,7 @@ void conv_hist(Tensor x, Tensor w, Tensor hist, Tensor row_item, Tensor cu, Tens
   const long long ss = hist_layout(hist, taps, C, "conv_hist hist");
   Items it = items_of(row_item, cu, item_slot, positions, hist.size(0), "conv_hist items");
   TORCH_CHECK(it.T == x.size(0), "conv_hist: one position per row");
+  TORCH_CHECK(!advance || it.n == it.T, "conv_hist: the fused history update wants items of one row");
   void* o2 = nullptr;
   int ldo2 = 0;
   if (out2.has_value()) {
@@ -335,7 +337,7 @@ void conv_hist(Tensor x, Tensor w, Tensor hist, Tensor row_item, Tensor cu, Tens
   }
   done(r32_conv_hist(x.data_ptr(), ldx, w.data_ptr<float>(), (int)w.stride(0), (int)w.stride(1), hist.data_ptr<float>(), ss,
                      it.row_item, it.cu, it.slot, it.pos,
-                     out.data_ptr(), ldo, o2, ldo2, it.T, C, taps, (int)mode, fi | (fo << 1), stream()), "conv_hist");
+                     out.data_ptr(), ldo, o2, ldo2, it.T, C, taps, (int)mode, fi | (fo << 1), advance ? 1 : 0, stream()), "conv_hist");
 }
 
 void conv_hist_update(Tensor x, Tensor hist, Tensor cu, Tensor item_slot, int64_t taps) {
@@ -535,8 +537,10 @@ std::vector<Tensor> router(Tensor z, Tensor corr, int64_t E, int64_t k) {
   const int T = (int)z.size(0), NE = (int)z.size(1);
   auto oi = z.options().dtype(torch::kInt32);
   Tensor ids = torch::empty({T, k}, oi), w = torch::empty({T, k}, z.options()), rank = torch::empty({T, k}, oi);
-  Tensor counts = torch::zeros({std::max<int64_t>(E, 1)}, oi), row_off = torch::empty({E + 1}, oi);
-  Tensor src = torch::zeros({T * k}, oi), row_expert = torch::zeros({T * k}, oi), inv = torch::empty({T * k}, oi);
+  const int64_t Ec = std::max<int64_t>(E, 1);
+  Tensor zeroed = torch::zeros({Ec + 2 * (int64_t)T * k}, oi);  // counts | src | row_expert: one fill
+  Tensor counts = zeroed.narrow(0, 0, Ec), src = zeroed.narrow(0, Ec, T * k), row_expert = zeroed.narrow(0, Ec + T * k, T * k);
+  Tensor row_off = torch::empty({E + 1}, oi), inv = torch::empty({T * k}, oi);
   done(r32_router(z.data_ptr<float>(), corr.data_ptr<float>(), T, NE, (int)E, (int)k, ids.data_ptr<int>(), w.data_ptr<float>(),
                   counts.data_ptr<int>(), rank.data_ptr<int>(), row_off.data_ptr<int>(), src.data_ptr<int>(),
                   row_expert.data_ptr<int>(), inv.data_ptr<int>(), stream()), "router");

@@ -20,19 +20,28 @@ namespace {
 
 template <typename IT, typename OT, int MODE>
 __global__ void conv_hist_kernel(const IT* __restrict__ x, int ldx, const float* __restrict__ w, int ws_c, int ws_j,
-                                 const float* __restrict__ hist, long long slot_stride, const int* __restrict__ row_item,
+                                 float* __restrict__ hist, long long slot_stride, const int* __restrict__ row_item,
                                  const int* __restrict__ cu, const int* __restrict__ item_slot,
                                  const int* __restrict__ positions, OT* __restrict__ out, int ldo, OT* __restrict__ out2,
-                                 int ldo2, int C, int taps) {
+                                 int ldo2, int C, int taps, int fuse) {
   const int t = blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= C) return;
   const int i = row_item[t];
   const int r = t - cu[i], p = positions[t];
-  const float* h = hist + (long long)item_slot[i] * slot_stride;
+  float* h = hist + (long long)item_slot[i] * slot_stride;
   const float cur = Elem<IT>::ld(x + (size_t)t * ldx + c);
   float acc = w[(size_t)c * ws_c + (size_t)(taps - 1) * ws_j] * cur;
-  for (int s = 1; s < taps; ++s) {
+  if (fuse) {  // every item is ONE row: this thread alone reads and rewrites its channel of the slot's history
+    for (int s = taps - 1; s >= 1; --s) {
+      const int e = taps - 1 - s;  // the entry that holds the input s rows back (meaningless before the start)
+      const float v = h[(size_t)e * C + c];
+      if (e >= 1) h[(size_t)(e - 1) * C + c] = v;
+      acc += w[(size_t)c * ws_c + (size_t)(taps - 1 - s) * ws_j] * (s <= p ? v : 0.f);
+    }
+    if (taps > 1) h[(size_t)(taps - 2) * C + c] = cur;
+  }
+  for (int s = 1; s < taps && !fuse; ++s) {
     float v = 0.f;
     if (s <= r) v = Elem<IT>::ld(x + (size_t)(t - s) * ldx + c);
     else if (s <= p) v = h[(size_t)(taps - 1 - (s - r)) * C + c];
@@ -49,19 +58,29 @@ __global__ void conv_hist_kernel(const IT* __restrict__ x, int ldx, const float*
 // Four channels per thread: weights stored tap-major (w[j][c]), every row base a multiple of four channels.
 template <typename IT, typename OT, int MODE>
 __global__ void conv_hist_vec_kernel(const IT* __restrict__ x, int ldx, const float* __restrict__ w,
-                                     const float* __restrict__ hist, long long slot_stride,
+                                     float* __restrict__ hist, long long slot_stride,
                                      const int* __restrict__ row_item, const int* __restrict__ cu,
                                      const int* __restrict__ item_slot, const int* __restrict__ positions,
-                                     OT* __restrict__ out, int ldo, OT* __restrict__ out2, int ldo2, int C, int taps) {
+                                     OT* __restrict__ out, int ldo, OT* __restrict__ out2, int ldo2, int C, int taps,
+                                     int fuse) {
   const int t = blockIdx.y;
   const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (c >= C) return;
   const int i = row_item[t];
   const int r = t - cu[i], p = positions[t];
-  const float* h = hist + (long long)item_slot[i] * slot_stride;
+  float* h = hist + (long long)item_slot[i] * slot_stride;
   const float4v cur = Vec4<IT>::ld(x + (size_t)t * ldx + c);
   float4v acc = Vec4<float>::ld(w + (size_t)(taps - 1) * C + c) * cur;
-  for (int s = 1; s < taps; ++s) {
+  if (fuse) {  // every item is ONE row: this thread alone reads and rewrites its channels of the slot's history
+    for (int s = taps - 1; s >= 1; --s) {
+      const int e = taps - 1 - s;
+      const float4v v = Vec4<float>::ld(h + (size_t)e * C + c);
+      if (e >= 1) Vec4<float>::st(h + (size_t)(e - 1) * C + c, v);
+      if (s <= p) acc += Vec4<float>::ld(w + (size_t)(taps - 1 - s) * C + c) * v;
+    }
+    if (taps > 1) Vec4<float>::st(h + (size_t)(taps - 2) * C + c, cur);
+  }
+  for (int s = 1; s < taps && !fuse; ++s) {
     float4v v = float4v{0.f, 0.f, 0.f, 0.f};
     if (s <= r) v = Vec4<IT>::ld(x + (size_t)(t - s) * ldx + c);
     else if (s <= p) v = Vec4<float>::ld(h + (size_t)(taps - 1 - (s - r)) * C + c);
@@ -284,10 +303,11 @@ using namespace lwc;
 
 // io: bit 0 = input fp32 (else bf16), bit 1 = output fp32 (else bf16)
 // w: element (c, j) at w[c * ws_c + j * ws_j]
-extern "C" int r32_conv_hist(const void* x, int ldx, const float* w, int ws_c, int ws_j, const float* hist,
+// fuse != 0: every item is one row (T == items) and the slot's history is advanced by the same kernel
+extern "C" int r32_conv_hist(const void* x, int ldx, const float* w, int ws_c, int ws_j, float* hist,
                              long long slot_stride, const int* row_item, const int* cu, const int* item_slot,
                              const int* positions, void* out, int ldo, void* out2, int ldo2, int T, int C, int taps,
-                             int mode, int io, hipStream_t s) {
+                             int mode, int io, int fuse, hipStream_t s) {
   if (T <= 0 || C <= 0) return 0;
   if (taps < 1 || taps > kMaxTaps) return -1;
   const int ib = (io & 1) ? 16 : 8, ob = (io & 2) ? 16 : 8;
@@ -300,11 +320,11 @@ extern "C" int r32_conv_hist(const void* x, int ldx, const float* w, int ws_c, i
   if (vec)                                                                                                             \
     conv_hist_vec_kernel<IT, OT, M><<<grid, threads, 0, s>>>((const IT*)x, ldx, w, hist, slot_stride, row_item, cu,   \
                                                              item_slot, positions, (OT*)out, ldo, (OT*)out2, ldo2, C, \
-                                                             taps);                                                    \
+                                                             taps, fuse);                                              \
   else                                                                                                                 \
     conv_hist_kernel<IT, OT, M><<<grid, threads, 0, s>>>((const IT*)x, ldx, w, ws_c, ws_j, hist, slot_stride,         \
                                                          row_item, cu, item_slot, positions, (OT*)out, ldo,            \
-                                                         (OT*)out2, ldo2, C, taps)
+                                                         (OT*)out2, ldo2, C, taps, fuse)
   if (mode == 0) {
     if (io == 3) {
       LWC_CONV(float, float, 0);

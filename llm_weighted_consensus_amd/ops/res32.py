@@ -137,15 +137,17 @@ class StepItems:
     [cu[i], cu[i+1]) at consecutive positions and the state slot ``slots[i]`` (a decode row is an item of one
     row).  All int32 device tensors; ``row_item[t]`` is the item of row t."""
 
-    def __init__(self, row_item: torch.Tensor, cu: torch.Tensor, slots: torch.Tensor, positions: torch.Tensor):
+    def __init__(self, row_item: torch.Tensor, cu: torch.Tensor, slots: torch.Tensor, positions: torch.Tensor,
+                 single: bool = False):
         self.row_item, self.cu, self.slots, self.positions = row_item, cu, slots, positions
+        self.single = single  # every item is one row: kernels may advance the state in the same pass
 
     @classmethod
     def rows(cls, slots: torch.Tensor, positions: torch.Tensor) -> "StepItems":
         """Every row its own item (a decode step); built from device tensors only (capturable)."""
         n = positions.numel()
         ar = torch.arange(n + 1, dtype=torch.int32, device=positions.device)
-        return cls(ar[:n], ar, slots, positions)
+        return cls(ar[:n], ar, slots, positions, single=True)
 
 
 def conv_hist(x: torch.Tensor, w: torch.Tensor, hist: torch.Tensor, items: StepItems, out: torch.Tensor,
@@ -155,8 +157,9 @@ def conv_hist(x: torch.Tensor, w: torch.Tensor, hist: torch.Tensor, items: StepI
     row's.  ``mode`` 0: out = x + conv(x) (``out2``: a copy of x in out's dtype); 1: out = silu(conv(x)).
     With ``update`` the slot then holds the last taps - 1 inputs after this step."""
     K = kernels()
-    K.conv_hist(x, w, hist, items.row_item, items.cu, items.slots, items.positions, out, out2, int(mode))
-    if update:
+    fused = bool(update and items.single)  # a decode step: one kernel computes and moves the history on
+    K.conv_hist(x, w, hist, items.row_item, items.cu, items.slots, items.positions, out, out2, int(mode), fused)
+    if update and not fused:
         K.conv_hist_update(x, hist, items.cu, items.slots, int(w.shape[1]))
     return out
 

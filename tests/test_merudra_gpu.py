@@ -71,6 +71,39 @@ def test_conv_with_history_in_portions(gpu, dtype, tol, taps, C, tap_major):
         assert (torch.cat(got["b"]).double() - rb).abs().max() < tol * 8
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 3e-2)])
+@pytest.mark.parametrize("taps,C,tap_major", [(1, 10, False), (3, 37, False), (4, 40, True)])
+def test_conv_decode_steps_advance_the_history_themselves(gpu, dtype, tol, taps, C, tap_major):
+    """Decode steps (every row its own sequence) compute and move the history on in ONE kernel: three sequences side
+    by side, one joining later behind a portion, against the oracle."""
+    from llm_weighted_consensus_amd.ops import res32
+
+    g = torch.Generator().manual_seed(taps + C)
+    n = 12
+    xs = [torch.randn(n, C, generator=g).to(dtype) for _ in range(3)]
+    w = torch.randn(C, taps, generator=g)
+    wg = w.to(gpu).t().contiguous().t() if tap_major else w.to(gpu)
+    refs = [x.double() + O.causal_conv(x.double(), w.double()) for x in xs]
+    hist = torch.randn(5, taps - 1, C, generator=g).to(gpu) * 50
+    slots = [3, 0, 4]
+    got = [[], [], []]
+    # sequence 2 starts with a portion of 5 rows (separate history update), then joins the decode steps
+    out = torch.empty(5, C, dtype=dtype, device=gpu)
+    res32.conv_hist(xs[2][:5].to(gpu), wg, hist, _items([5], [slots[2]], [0], gpu), out)
+    got[2].append(out.cpu())
+    for t in range(n):
+        who = [0, 1] + ([2] if t >= 5 else [])
+        x = torch.stack([xs[k][t] for k in who]).to(gpu)
+        items = res32.StepItems.rows(torch.tensor([slots[k] for k in who], dtype=torch.int32, device=gpu),
+                                     torch.full((len(who),), t, dtype=torch.int32, device=gpu))
+        out = torch.empty(len(who), C, dtype=dtype, device=gpu)
+        res32.conv_hist(x, wg, hist, items, out)
+        for j, k in enumerate(who):
+            got[k].append(out[j:j + 1].cpu())
+    for k in range(3):
+        assert (torch.cat(got[k]).double() - refs[k]).abs().max() < tol * 8
+
+
 @pytest.mark.parametrize("H,G,D,Dv", [(4, 2, 12, 20), (2, 2, 64, 64), (3, 1, 80, 72), (2, 1, 130, 8)])
 def test_delta_rule_whole_portions_and_single_tokens(gpu, H, G, D, Dv):
     """The gated delta rule of the kernel (unit q / k, decay, beta, state carried in a slot) against the oracle's
