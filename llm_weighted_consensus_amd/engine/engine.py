@@ -439,9 +439,10 @@ class LLMEngine:
         if len(prompt_ids) + params.max_tokens > self.max_model_len:
             raise ValueError(f"prompt ({len(prompt_ids)}) + max_tokens ({params.max_tokens}) exceeds "
                              f"max_model_len ({self.max_model_len})")
-        if prefilled is not None and self.state is not None:
+        state = getattr(self, "state", None)
+        if prefilled is not None and state is not None:
             raise ValueError("a prompt prefilled elsewhere brings no recurrent state")
-        if self.state is not None and n > self.max_batch:
+        if state is not None and n > self.max_batch:
             raise ValueError("n exceeds the number of recurrent-state slots (max_batch)")
         g = SequenceGroup(self, list(prompt_ids), params, n, callback)
         g.prefilled = prefilled
