@@ -66,6 +66,47 @@ __global__ void head_norm_kv_write_kernel(const AT* __restrict__ proj, int ldp, 
   }
 }
 
+// D / 4 (and Dv / 4) a power of two <= 64, every base a multiple of four elements: LPH = D / 4 lanes per head and
+// 64 / LPH heads per wave at once; 8- / 16-byte loads and stores except the interleaved value stores.
+template <typename AT>
+__global__ void head_norm_kv_write_sub_kernel(const AT* __restrict__ proj, int ldp, int k_off, int v_off,
+                                              const int* __restrict__ positions, const int* __restrict__ slots,
+                                              float* __restrict__ q_out, AT* __restrict__ k_cache, AT* __restrict__ v_cache,
+                                              long long kb_stride, long long vb_stride, int block_size, int H, int G, int D,
+                                              float eps, float scale, float coef, int every, int LPH) {
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const int hpw = 64 / LPH, sub = lane / LPH, i = (lane - sub * LPH) * 4;
+  const AT* pr = proj + (size_t)t * ldp;
+  const int p = positions[t];
+  const float qmul = scale * (1.0f + (every > 0 ? coef * logf((float)((p + 1) / every) + 1.0f) : 0.f));
+  const int slot = slots[t];
+  const bool write = slot >= 0;
+  const long long blk = write ? slot / block_size : 0, off = write ? slot % block_size : 0;
+  const int nk = G * D;
+  for (int h0 = wv * hpw; h0 < H + G; h0 += nw * hpw) {
+    const int h = h0 + sub;
+    const bool ok = h < H + G, isq = h < H;
+    const AT* src = !ok ? pr : (isq ? pr + h * D : pr + k_off + (h - H) * D);
+    const float4v v = Vec4<AT>::ld(src + i);
+    float s = v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+    for (int m = LPH >> 1; m > 0; m >>= 1) s += __shfl_xor(s, m, 64);
+    const float rstd = 1.0f / sqrtf(s / (float)D + eps);
+    if (!ok) continue;
+    if (isq) {
+      Vec4<float>::st(q_out + (size_t)t * H * D + h * D + i, v * (rstd * qmul));
+    } else if (write) {
+      const int g = h - H;
+      Vec4<AT>::st(k_cache + blk * kb_stride + off * nk + g * D + i, v * rstd);
+      // V is 4-token interleaved: [block][offset / 4][column][offset % 4]; here the values are D wide like the keys
+      AT* vc = v_cache + blk * vb_stride + (off >> 2) * (4LL * nk) + (off & 3) + 4LL * (g * D + i);
+      const AT* vs = pr + v_off + g * D + i;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) vc[4 * e] = vs[e];
+    }
+  }
+}
+
 template <typename AT, int MODE>
 __global__ void gate_mul_kernel(AT* __restrict__ a, int lda, const AT* __restrict__ g, int ldg, int n, long long total) {
   for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (long long)gridDim.x * blockDim.x) {
@@ -218,6 +259,20 @@ extern "C" int r32_head_norm_kv_write(const void* proj, int ldp, int k_off, int 
                                       long long vb_stride, int block_size, int T, int H, int G, int D, int Dv, float eps,
                                       float scale, float coef, int every, int f32, hipStream_t s) {
   if (T <= 0) return 0;
+  const int lph = D / 4, ab = f32 ? 16 : 8;
+  if (D == Dv && D % 4 == 0 && lph <= 64 && (lph & (lph - 1)) == 0 && ldp % 4 == 0 && k_off % 4 == 0 && v_off % 4 == 0 &&
+      kb_stride % 4 == 0 && aligned_to(proj, ab) && aligned_to(k_cache, ab) && aligned_to(q_out, 16)) {
+    if (f32)
+      head_norm_kv_write_sub_kernel<float><<<T, 256, 0, s>>>((const float*)proj, ldp, k_off, v_off, positions, slots, q_out,
+                                                              (float*)k_cache, (float*)v_cache, kb_stride, vb_stride,
+                                                              block_size, H, G, D, eps, scale, coef, every, lph);
+    else
+      head_norm_kv_write_sub_kernel<bf16_t><<<T, 256, 0, s>>>((const bf16_t*)proj, ldp, k_off, v_off, positions, slots,
+                                                               q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, kb_stride,
+                                                               vb_stride, block_size, H, G, D, eps, scale, coef, every, lph);
+    LWC_CHECK_LAUNCH();
+    return 0;
+  }
   if (f32)
     head_norm_kv_write_kernel<float><<<T, 256, 0, s>>>((const float*)proj, ldp, k_off, v_off, positions, slots, q_out,
                                                         (float*)k_cache, (float*)v_cache, kb_stride, vb_stride, block_size, H,

@@ -94,6 +94,54 @@ __global__ void conv_hist_vec_kernel(const IT* __restrict__ x, int ldx, const fl
   }
 }
 
+// Four channels x R consecutive rows per thread (taps <= 8): a row's earlier inputs stay in registers from the rows
+// before it, so x is read about once instead of `taps` times and the weights once per thread.
+template <typename IT, typename OT, int MODE, int R>
+__global__ void conv_hist_tile_kernel(const IT* __restrict__ x, int ldx, const float* __restrict__ w,
+                                      const float* __restrict__ hist, long long slot_stride,
+                                      const int* __restrict__ row_item, const int* __restrict__ cu,
+                                      const int* __restrict__ item_slot, const int* __restrict__ positions,
+                                      OT* __restrict__ out, int ldo, OT* __restrict__ out2, int ldo2, int C, int taps,
+                                      int T) {
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (c >= C) return;
+  const int t0 = blockIdx.y * R;
+  const float4v zero = float4v{0.f, 0.f, 0.f, 0.f};
+  float4v wv[8], prev[7];  // wv[s]: the weight of the input s rows back; prev[s - 1]: that input
+#pragma unroll
+  for (int s = 0; s < 8; ++s) wv[s] = s < taps ? Vec4<float>::ld(w + (size_t)(taps - 1 - s) * C + c) : zero;
+#pragma unroll
+  for (int s = 1; s < 8; ++s) prev[s - 1] = (s < taps && t0 - s >= 0) ? Vec4<IT>::ld(x + (size_t)(t0 - s) * ldx + c) : zero;
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    const int t = t0 + j;
+    if (t >= T) break;
+    const int i = row_item[t];
+    const int r = t - cu[i], p = positions[t];
+    const float* h = hist + (long long)item_slot[i] * slot_stride;
+    const float4v cur = Vec4<IT>::ld(x + (size_t)t * ldx + c);
+    float4v acc = wv[0] * cur;
+#pragma unroll
+    for (int s = 1; s < 8; ++s) {
+      if (s < taps) {
+        float4v v = zero;
+        if (s <= r) v = prev[s - 1];
+        else if (s <= p) v = Vec4<float>::ld(h + (size_t)(taps - 1 - (s - r)) * C + c);
+        acc += wv[s] * v;
+      }
+    }
+    if (MODE == 0) {
+      Vec4<OT>::st(out + (size_t)t * ldo + c, cur + acc);
+      if (out2) Vec4<OT>::st(out2 + (size_t)t * ldo2 + c, cur);
+    } else {
+      Vec4<OT>::st(out + (size_t)t * ldo + c, float4v{silu_f(acc[0]), silu_f(acc[1]), silu_f(acc[2]), silu_f(acc[3])});
+    }
+#pragma unroll
+    for (int s = 6; s >= 1; --s) prev[s] = prev[s - 1];
+    prev[0] = cur;
+  }
+}
+
 constexpr int kMaxTaps = 16;
 
 template <typename IT>
@@ -296,6 +344,35 @@ __global__ void head_norm_gate_vec_kernel(const float* __restrict__ o, int ldi, 
   }
 }
 
+// Dv / 4 a power of two <= 64: LPH = Dv / 4 lanes per head, 64 / LPH heads per wave at once, every lane busy
+template <typename AT, int GATE>
+__global__ void head_norm_gate_sub_kernel(const float* __restrict__ o, int ldi, const AT* __restrict__ gate, int ldg,
+                                          const float* __restrict__ w, AT* __restrict__ out, int ldo, int H, int Dv,
+                                          float eps, int LPH) {
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const int hpw = 64 / LPH, sub = lane / LPH, i = (lane - sub * LPH) * 4;
+  for (int h0 = wv * hpw; h0 < H; h0 += nw * hpw) {
+    const int h = h0 + sub;
+    const bool ok = h < H;
+    const float* oh = o + (size_t)t * ldi + (ok ? h : 0) * Dv;
+    const float4v v = Vec4<float>::ld(oh + i);
+    float s = v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+    for (int m = LPH >> 1; m > 0; m >>= 1) s += __shfl_xor(s, m, 64);
+    const float rstd = 1.0f / sqrtf(s / (float)Dv + eps);
+    float4v y = v * rstd;
+    if (w) y *= Vec4<float>::ld(w + i);
+    if (ok) {
+      if (GATE) {
+        const float4v z = Vec4<AT>::ld(gate + (size_t)t * ldg + h * Dv + i);
+        y *= GATE == 1 ? float4v{silu_f(z[0]), silu_f(z[1]), silu_f(z[2]), silu_f(z[3])}
+                       : float4v{sigmoid_f(z[0]), sigmoid_f(z[1]), sigmoid_f(z[2]), sigmoid_f(z[3])};
+      }
+      Vec4<AT>::st(out + (size_t)t * ldo + h * Dv + i, y);
+    }
+  }
+}
+
 }  // namespace
 }  // namespace lwc
 
@@ -314,10 +391,17 @@ extern "C" int r32_conv_hist(const void* x, int ldx, const float* w, int ws_c, i
   const bool vec = ws_c == 1 && (taps == 1 || ws_j == C) && C % 4 == 0 && ldx % 4 == 0 && ldo % 4 == 0 && ldo2 % 4 == 0 &&
                    slot_stride % 4 == 0 && aligned_to(x, ib) && aligned_to(out, ob) && aligned_to(out2, ob) &&
                    aligned_to(w, 16) && aligned_to(hist, 16);
-  dim3 grid(vec ? (C / 4 + 63) / 64 : (C + 255) / 256, T);
-  const int threads = vec ? 64 : 256;
+  const int threads = vec && C / 4 <= 64 ? 64 : (vec && C / 4 <= 128 ? 128 : 256);
+  dim3 grid(vec ? (C / 4 + threads - 1) / threads : (C + 255) / 256, T);
+  constexpr int kRows = 8;
+  const bool tile = vec && !fuse && taps <= 8 && T >= 8 * kRows;
+  dim3 tgrid(grid.x, (T + kRows - 1) / kRows);
 #define LWC_CONV(IT, OT, M)                                                                                            \
-  if (vec)                                                                                                             \
+  if (tile)                                                                                                            \
+    conv_hist_tile_kernel<IT, OT, M, kRows><<<tgrid, threads, 0, s>>>((const IT*)x, ldx, w, hist, slot_stride,        \
+                                                                       row_item, cu, item_slot, positions, (OT*)out,  \
+                                                                       ldo, (OT*)out2, ldo2, C, taps, T);             \
+  else if (vec)                                                                                                        \
     conv_hist_vec_kernel<IT, OT, M><<<grid, threads, 0, s>>>((const IT*)x, ldx, w, hist, slot_stride, row_item, cu,   \
                                                              item_slot, positions, (OT*)out, ldo, (OT*)out2, ldo2, C, \
                                                              taps, fuse);                                              \
@@ -407,8 +491,13 @@ extern "C" int r32_head_norm_gate(const float* o, int ldi, const void* gate, int
   const int ab = f32 ? 16 : 8;
   const bool vec = Dv % 4 == 0 && ldi % 4 == 0 && ldg % 4 == 0 && ldo % 4 == 0 && aligned_to(o, 16) && aligned_to(w, 16) &&
                    aligned_to(gate, ab) && aligned_to(out, ab);
+  const int lph = Dv / 4;
+  const bool sub = vec && lph >= 1 && lph <= 64 && (lph & (lph - 1)) == 0;
 #define LWC_HNG(AT, GM)                                                                                                  \
-  if (vec)                                                                                                               \
+  if (sub)                                                                                                               \
+    head_norm_gate_sub_kernel<AT, GM><<<T, threads, 0, s>>>(o, ldi, (const AT*)gate, ldg, w, (AT*)out, ldo, H, Dv, eps,  \
+                                                            lph);                                                        \
+  else if (vec)                                                                                                          \
     head_norm_gate_vec_kernel<AT, GM><<<T, threads, 0, s>>>(o, ldi, (const AT*)gate, ldg, w, (AT*)out, ldo, H, Dv, eps); \
   else                                                                                                                   \
     head_norm_gate_kernel<AT, GM><<<T, threads, 0, s>>>(o, ldi, (const AT*)gate, ldg, w, (AT*)out, ldo, H, Dv, eps)

@@ -72,6 +72,37 @@ def test_conv_with_history_in_portions(gpu, dtype, tol, taps, C, tap_major):
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 3e-2)])
+@pytest.mark.parametrize("taps,C", [(4, 40), (2, 264), (8, 12), (9, 12)])
+def test_conv_many_rows_of_several_sequences(gpu, dtype, tol, taps, C):
+    """A step of 128 rows of three sequences that each continue behind a short first portion (the kernel that keeps a
+    row's earlier inputs in registers takes it for up to 8 taps): item borders inside a thread's rows, histories
+    read at the borders, against the oracle."""
+    from llm_weighted_consensus_amd.ops import res32
+
+    g = torch.Generator().manual_seed(taps * 7 + C)
+    lens, first = [60, 45, 33], [7, 2, 1]
+    xs = [torch.randn(n, C, generator=g).to(dtype) for n in lens]
+    w = torch.randn(C, taps, generator=g)
+    wg = w.to(gpu).t().contiguous().t()
+    hist = torch.randn(4, taps - 1, C, generator=g).to(gpu) * 50
+    slots = [1, 3, 0]
+    for mode in (0, 1):
+        refs = [O.causal_conv(x.double(), w.double()) for x in xs]
+        refs = [x.double() + y if mode == 0 else O.silu(y) for x, y in zip(xs, refs)]
+        x1 = torch.cat([x[:f] for x, f in zip(xs, first)]).to(gpu)
+        o1 = torch.empty(x1.shape[0], C, dtype=dtype, device=gpu)
+        res32.conv_hist(x1, wg, hist, _items(first, slots, [0, 0, 0], gpu), o1, mode=mode)
+        x2 = torch.cat([x[f:] for x, f in zip(xs, first)]).to(gpu)
+        o2 = torch.empty(x2.shape[0], C, dtype=dtype, device=gpu)
+        res32.conv_hist(x2, wg, hist, _items([n - f for n, f in zip(lens, first)], slots, first, gpu), o2, mode=mode)
+        a1 = a2 = 0
+        for k, (n, f) in enumerate(zip(lens, first)):
+            got = torch.cat([o1[a1:a1 + f], o2[a2:a2 + n - f]]).cpu().double()
+            assert (got - refs[k]).abs().max() < tol * 10, (mode, k)
+            a1, a2 = a1 + f, a2 + n - f
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 3e-2)])
 @pytest.mark.parametrize("taps,C,tap_major", [(1, 10, False), (3, 37, False), (4, 40, True)])
 def test_conv_decode_steps_advance_the_history_themselves(gpu, dtype, tol, taps, C, tap_major):
     """Decode steps (every row its own sequence) compute and move the history on in ONE kernel: three sequences side
@@ -144,11 +175,12 @@ def test_delta_rule_whole_portions_and_single_tokens(gpu, H, G, D, Dv):
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 3e-2)])
-def test_head_norm_gate_and_gated_norm_residual(gpu, dtype, tol):
+@pytest.mark.parametrize("H,Dv", [(3, 20), (5, 32), (9, 128), (2, 7)])
+def test_head_norm_gate_and_gated_norm_residual(gpu, dtype, tol, H, Dv):
     from llm_weighted_consensus_amd.ops import res32
 
     g = torch.Generator().manual_seed(5)
-    T, H, Dv, d = 7, 3, 20, 52
+    T, d = 7, 52
     o = torch.randn(T, H * Dv, generator=g) * 3
     gate = torch.randn(T, H * Dv + 6, generator=g).to(dtype)
     w = 1 + 0.2 * torch.randn(Dv, generator=g)
@@ -235,7 +267,7 @@ def test_head_norm_cache_write_and_attention(gpu, dtype, tol, H, G, D, every):
     g = torch.Generator().manual_seed(H + D)
     n, bs, scale, coef, eps = 45, 16, 0.37, 0.6, 1e-4
     nq, nk = H * D, G * D
-    proj = (torch.randn(n, nq + nk + 3, generator=g) * 2).to(dtype)
+    proj = (torch.randn(n, nq + nk + (4 if D % 16 == 0 else 3), generator=g) * 2).to(dtype)  # (row stride: both kernels)
     q, k = proj[:, :nq].double().view(n, H, D), proj[:, nq:nq + nk].double().view(n, G, D)
     qn = O.rms_unit(q, eps) * O.query_temperature(range(n), coef, every)[:, None, None]
     ref = O.softmax_attention(qn, O.rms_unit(k, eps), k, H, G, scale)
