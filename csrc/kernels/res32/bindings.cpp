@@ -378,7 +378,7 @@ void delta_rule(Tensor qkv, Tensor ba, int64_t b_off, int64_t a_off, Tensor A_lo
                   ba.size(0) == T && b_off >= 0 && a_off >= 0 && b_off + H <= ba.size(1) && a_off + H <= ba.size(1) &&
                   A_log.numel() == H && dt_bias.numel() == H && positions.numel() == T && cu.numel() == item_slot.numel() + 1 &&
                   D <= r32_delta_rule_max_dim(), "delta_rule: shapes disagree");
-  Tensor bg = torch::empty({T, 2 * H}, qkv.options());
+  Tensor bg = torch::empty({T, 2 * H + G}, qkv.options());
   done(r32_delta_rule(qkv.data_ptr<float>(), ldq, ba.data_ptr(), ldb, (int)b_off, (int)a_off, A_log.data_ptr<float>(),
                       dt_bias.data_ptr<float>(), bg.data_ptr<float>(), state.data_ptr<float>(), (long long)state.stride(0),
                       cu.data_ptr<int>(), item_slot.data_ptr<int>(), positions.data_ptr<int>(), out.data_ptr<float>(), ldo, T,

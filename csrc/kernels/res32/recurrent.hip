@@ -173,8 +173,8 @@ __global__ void conv_hist_update_kernel(const IT* __restrict__ x, int ldx, float
 }
 
 // Before the recurrence, per row and in parallel over rows: q and k (fp32 rows [q (G*D) | k (G*D) | v (H*Dv)]) made
-// unit vectors per head IN PLACE (q also times D^-1/2), and bg[t] = [beta_h | decay_h] from the projection columns
-// ba[:, b_off + h], ba[:, a_off + h].
+// unit vectors per head IN PLACE (q also times D^-1/2), and bg[t] = [beta_h | decay_h | (q . k)_g] with beta and the
+// decay from the projection columns ba[:, b_off + h], ba[:, a_off + h].
 template <typename AT>
 __global__ void delta_prep_kernel(float* __restrict__ qkv, int ldq, const AT* __restrict__ ba, int ldb, int b_off,
                                   int a_off, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
@@ -189,9 +189,19 @@ __global__ void delta_prep_kernel(float* __restrict__ qkv, int ldq, const AT* __
     const float r = (v < G ? qscale : 1.0f) / sqrtf(wave_sum(s) + 1e-6f);
     for (int i = lane; i < D; i += 64) x[i] *= r;
   }
+  const int nb = 2 * H + G;  // bg row: beta_h | decay_h | (q . k)_g
   for (int h = threadIdx.x; h < H; h += blockDim.x) {
-    bg[(size_t)t * 2 * H + h] = sigmoid_f(Elem<AT>::ld(ba + (size_t)t * ldb + b_off + h));
-    bg[(size_t)t * 2 * H + H + h] = expf(-expf(A_log[h]) * softplus_f(Elem<AT>::ld(ba + (size_t)t * ldb + a_off + h) + dt_bias[h]));
+    bg[(size_t)t * nb + h] = sigmoid_f(Elem<AT>::ld(ba + (size_t)t * ldb + b_off + h));
+    bg[(size_t)t * nb + H + h] = expf(-expf(A_log[h]) * softplus_f(Elem<AT>::ld(ba + (size_t)t * ldb + a_off + h) + dt_bias[h]));
+  }
+  __syncthreads();  // the normalised q and k of this row are written
+  for (int g = wv; g < G; g += nw) {
+    const float* q = qkv + (size_t)t * ldq + (size_t)g * D;
+    const float* k = q + (size_t)G * D;
+    float s = 0.f;
+    for (int i = lane; i < D; i += 64) s += q[i] * k[i];
+    s = wave_sum(s);
+    if (lane == 0) bg[(size_t)t * nb + 2 * H + g] = s;
   }
 }
 
@@ -224,67 +234,75 @@ __global__ void __launch_bounds__(64 * NW) delta_rule_kernel(const float* __rest
 #pragma unroll
   for (int j = 0; j < DPL; ++j) S[j] = (i0 + j < D && live && !fresh) ? Sg[(size_t)j * Dv] : 0.f;
   const int nq = G * D;
-  float stage[PER], vn = 0.f, bn = 0.f, gn = 0.f;
-  auto fetch = [&](int row) {  // the row's k and q chunk of this thread, its value, beta and decay -> registers
+  // a token's operands in registers on their way to LDS: its chunk of k and q, its value, beta, decay and q . k
+  struct Stage {
+    float kq[PER], v, beta, g, qk;
+  };
+  const int nb = 2 * H + G;
+  auto fetch = [&](int row, Stage& st) {
     const float* qr = qkv + (size_t)row * ldq + kvh * D;
 #pragma unroll
     for (int u = 0; u < PER; ++u) {
       const int e = tid + 64 * NW * u;       // e < 4 DPL: k row e; else q row e - 4 DPL
       const int which = e >= 4 * DPL, i = e - which * 4 * DPL;
-      stage[u] = (e < 8 * DPL && i < D) ? qr[(which ? 0 : nq) + i] : 0.f;
+      st.kq[u] = (e < 8 * DPL && i < D) ? qr[(which ? 0 : nq) + i] : 0.f;
     }
-    vn = live ? qkv[(size_t)row * ldq + 2 * nq + h * Dv + col] : 0.f;
-    bn = bg[(size_t)row * 2 * H + h];
-    gn = bg[(size_t)row * 2 * H + H + h];
+    st.v = live ? qkv[(size_t)row * ldq + 2 * nq + h * Dv + col] : 0.f;
+    st.beta = bg[(size_t)row * nb + h];
+    st.g = bg[(size_t)row * nb + H + h];
+    st.qk = bg[(size_t)row * nb + 2 * H + kvh];
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](int buf, const Stage& st) {
 #pragma unroll
     for (int u = 0; u < PER; ++u) {
       const int e = tid + 64 * NW * u;
       const int which = e >= 4 * DPL, i = e - which * 4 * DPL;
-      if (e < 8 * DPL) kq_s[buf][which][(i / DPL) * QLD + i % DPL] = stage[u];
+      if (e < 8 * DPL) kq_s[buf][which][(i / DPL) * QLD + i % DPL] = st.kq[u];
     }
   };
-  fetch(r0);
-  stash(0);
-  float v = vn, beta = bn, g = gn;
+  // Two register stages alternate, so a token's loads are issued two tokens before they are needed (one token's
+  // arithmetic is shorter than a trip to memory).
+  Stage A, B;
+  fetch(r0, A);
+  stash(0, A);
+  float v = A.v, beta = A.beta, g = A.g, qk = A.qk;
+  if (r0 + 1 < r1) fetch(r0 + 1, A);
+  if (r0 + 2 < r1) fetch(r0 + 2, B);
   __syncthreads();
-  for (int row = r0; row < r1; ++row) {
-    const int cur = (row - r0) & 1;
-    if (row + 1 < r1) fetch(row + 1);
+  // one token out of LDS buffer `cur`; `next` holds the following token's operands and is refilled three ahead
+  auto step = [&](int row, int cur, Stage& next) {
     const float4v* ks = reinterpret_cast<const float4v*>(&kq_s[cur][0][r * QLD]);
     const float4v* qs = reinterpret_cast<const float4v*>(&kq_s[cur][1][r * QLD]);
+    // With S the state BEFORE this token: S^T k and S^T q in one pass (independent partial sums), then
+    //   u = beta (v - g S^T k),   o = (g S + k u^T)^T q = g S^T q + (k . q) u,   S <- g S + k u^T
     float kk[DPL];
-    float dot = 0.f;
+    float4v dk = float4v{0.f, 0.f, 0.f, 0.f}, dq = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < DPL / 4; ++j) {
-      const float4v k4 = ks[j];
+      const float4v k4 = ks[j], q4 = qs[j];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         kk[4 * j + e] = k4[e];
-        S[4 * j + e] *= g;
-        dot += S[4 * j + e] * k4[e];
+        dk[e] += S[4 * j + e] * k4[e];
+        dq[e] += S[4 * j + e] * q4[e];
       }
     }
-    dot = row_sum4(dot);
-    const float u = beta * (v - dot);
-    float o = 0.f;
+    const float sk = row_sum4((dk[0] + dk[1]) + (dk[2] + dk[3]));
+    const float sq = row_sum4((dq[0] + dq[1]) + (dq[2] + dq[3]));
+    const float u = beta * (v - g * sk);
+    if (live && r == 0) out[(size_t)row * ldo + h * Dv + col] = g * sq + qk * u;
 #pragma unroll
-    for (int j = 0; j < DPL / 4; ++j) {
-      const float4v q4 = qs[j];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        S[4 * j + e] += kk[4 * j + e] * u;
-        o += S[4 * j + e] * q4[e];
-      }
-    }
-    o = row_sum4(o);
-    if (live && r == 0) out[(size_t)row * ldo + h * Dv + col] = o;
+    for (int j = 0; j < DPL; ++j) S[j] = kk[j] * u + g * S[j];
     if (row + 1 < r1) {
-      stash(cur ^ 1);
-      v = vn, beta = bn, g = gn;
+      stash(cur ^ 1, next);
+      v = next.v, beta = next.beta, g = next.g, qk = next.qk;
+      if (row + 3 < r1) fetch(row + 3, next);
     }
     __syncthreads();
+  };
+  for (int row = r0; row < r1; row += 2) {
+    step(row, 0, A);
+    if (row + 1 < r1) step(row + 1, 1, B);
   }
   if (live) {
 #pragma unroll
@@ -448,7 +466,7 @@ extern "C" int r32_conv_hist_update(const void* x, int ldx, float* hist, long lo
 
 extern "C" int r32_delta_rule_max_dim() { return 256; }
 
-// qkv is normalised in place (q, k columns); bg fp32 [T, 2 H] scratch for beta and the decays
+// qkv is normalised in place (q, k columns); bg fp32 [T, 2 H + G] scratch for beta, the decays and q . k
 extern "C" int r32_delta_rule(float* qkv, int ldq, const void* ba, int ldb, int b_off, int a_off, const float* A_log,
                               const float* dt_bias, float* bg, float* state, long long slot_stride, const int* cu,
                               const int* item_slot, const int* positions, float* out, int ldo, int T, int items, int H,
