@@ -355,6 +355,14 @@ class LLMEngine:
             raise ValueError("chunked prefill: the paged-KV prefill kernel is built for head_dim 128")
         self.prefilling: List[SequenceGroup] = []
         self.width = (max_model_len + block_size - 1) // block_size
+        # models with recurrent layers: one state slot per live sequence, handed out by the block manager with the
+        # sequence's blocks (models/state.py); the pool's last slot is scratch for padded rows and warm-up runs.
+        # Allocated before the KV pool is sized from the memory that is left.
+        self.state = None
+        if getattr(model, "has_state", False):
+            if prefix_caching:
+                raise ValueError("prefix caching cannot skip a prompt's head for a model with recurrent state")
+            self.state = model.new_state(max_batch)
         if num_blocks is None:
             free, _total = torch.cuda.mem_get_info(self.device)
             per = (model.bytes_per_block(block_size) if hasattr(model, "bytes_per_block")
@@ -364,13 +372,7 @@ class LLMEngine:
         self.cache = (model.new_cache(num_blocks, block_size) if hasattr(model, "new_cache")
                       else KVCache(self.cfg, num_blocks, block_size, self.device))
         self.bm = BlockManager(num_blocks, block_size)
-        # models with recurrent layers: one state slot per live sequence, handed out by the block manager with the
-        # sequence's blocks (models/state.py); the pool's last slot is scratch for padded rows and warm-up runs
-        self.state = None
-        if getattr(model, "has_state", False):
-            if prefix_caching:
-                raise ValueError("prefix caching cannot skip a prompt's head for a model with recurrent state")
-            self.state = model.new_state(max_batch)
+        if self.state is not None:
             self.bm.set_state_slots(max_batch)
         # cross-request prefix cache (C++ block manager): prompts that start with an already computed
         # token prefix (the shared messages of a score request's voters, a repeated conversation) reuse

@@ -777,7 +777,8 @@ def build_engine(spec: dict, wid: int):
     return LLMEngine(model, tok, max_batch=int(spec.get("max_batch", 512)), max_model_len=mlen,
                      kv_memory_fraction=kv_fraction, num_blocks=num_blocks,
                      use_graphs=getattr(model, "graph_safe", True),
-                     prefix_caching=bool(spec.get("prefix_caching", True)),
+                     # (a prompt's cached head brings no recurrent state: off for models that carry one)
+                     prefix_caching=bool(spec.get("prefix_caching", True)) and not getattr(model, "has_state", False),
                      # the paged-KV prefill kernel of mixed steps is built for head_dim 128
                      chunked_prefill=(int(spec.get("chunked_prefill", 0))
                                       if cfg.head_dim == 128 or getattr(model, "paged_prefill", False) else 0),

@@ -624,6 +624,27 @@ def test_preemption_keeps_the_recurrent_state(gpu, tmp_path):
     assert eng.bm.num_free == eng.bm.num_blocks and eng.bm.num_free_state_slots == 4
 
 
+def test_server_worker_factory_builds_the_design(gpu, tmp_path):
+    """The server's worker factory (`engine.group.build_engine`) on a model folder of the design: prefix caching is
+    switched off for it (a cached head brings no recurrent state), the state pool is there, generation works."""
+    from safetensors.torch import save_file
+
+    from llm_weighted_consensus_amd.engine.group import build_engine
+    from llm_weighted_consensus_amd.engine.sampling import SamplingParams
+
+    c = CONFIGS["cores"]
+    cfg = O.make_config(c["width"], c["vocab"], c["layers"], taps=c["taps"], side=c["side"])
+    W = O.make_weights(cfg, 2)
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.contiguous() for k, v in W.items()}, str(tmp_path / "model.safetensors"))
+    eng = build_engine({"model_dir": str(tmp_path), "dtype": "float32", "max_batch": 4, "max_model_len": 128,
+                        "kv_fraction": 0.001}, 0)
+    assert eng.state is not None and not eng.prefix_caching and eng.bm.num_state_slots == 4
+    prompt = _tokens(20, cfg["vocab"], 8)
+    out = eng.generate([prompt], SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))
+    _check_greedy(cfg, W, prompt, out[0][0])
+
+
 def test_trace_replay_command_line(gpu, tmp_path):
     """bin/trace_run as a user runs it: JSON lines in, ``done <step>`` lines and <step>.f32 files out; two sequences
     interleaved (portions beside single tokens, one sitting a step out), pages and slots given back at ``end``."""
